@@ -128,6 +128,19 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
  * pa_attention ignores key/value). */
 int32_t pa_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
+/* pa_attention for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as pa_attention, for steps
+ * in which every sequence schedules one token, over a u8 cache or a 16-bit cache of the query's type (block size 32,
+ * head size 64 or 128, at most 16 query heads per kv head); other steps return PA_NOT_IMPLEMENTED.  The split partials,
+ * final maxima / denominators and the score staging live in a fixed device array of PA_STATIC_SCRATCH_BYTES bytes
+ * (32 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls
+ * no hipMalloc / hipFree; a step that needs more returns PA_OUT_OF_BOUNDS and a message with the byte count.  (The
+ * step arrays and block tables are uploaded -- and their buffers grown -- by pa_step_begin / pa_set_block_indices,
+ * as for pa_attention.)  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race, also from
+ * different contexts; calls in stream order on one stream do not.  Nothing in it needs clearing between calls: each
+ * call writes every element it later reads. */
+#define PA_STATIC_SCRATCH_BYTES (32u << 20)
+int32_t pa_attention_static(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* Blocks until everything launched on the context's stream has finished. */
 int32_t pa_synchronize(pa_ctx* ctx);
 /* Number of split-K partitions of the last attention call (diagnostics). */

@@ -10,6 +10,7 @@ SO_PATH = os.path.join(_HERE, "csrc", "libpa_amd.so")
 
 PA_OK = 0
 PA_F16, PA_BF16, PA_U8 = 0, 1, 2
+PA_STATIC_SCRATCH_BYTES = 32 << 20
 PA_AGG_SUM, PA_AGG_NORM_SUM, PA_AGG_ADAPTIVE_RKV = 0, 1, 2
 (PA_KVCRUSH_ANCHOR_RANDOM, PA_KVCRUSH_ANCHOR_ZEROS, PA_KVCRUSH_ANCHOR_ONES, PA_KVCRUSH_ANCHOR_MEAN,
  PA_KVCRUSH_ANCHOR_ALTERNATING) = range(5)
@@ -20,7 +21,7 @@ STATUS_NAMES = {0: "OK", -1: "GENERAL_ERROR", -2: "NOT_IMPLEMENTED", -4: "PARAME
 # every symbol include/pa_amd.h declares
 EXPORTS = [
     "pa_version", "pa_global_last_error", "pa_create", "pa_destroy", "pa_last_error", "pa_step_begin",
-    "pa_set_block_indices", "pa_forward", "pa_kv_append", "pa_attention", "pa_synchronize", "pa_get_num_splits", "pa_set_profiling", "pa_last_kernel_ms",
+    "pa_set_block_indices", "pa_forward", "pa_kv_append", "pa_attention", "pa_attention_static", "pa_synchronize", "pa_get_num_splits", "pa_set_profiling", "pa_last_kernel_ms",
     "pa_pack_step", "pa_snapkv_num_scores", "pa_kv_cache_create", "pa_kv_cache_destroy", "pa_kv_cache_last_error",
     "pa_kv_cache_block_bytes", "pa_kv_cache_allocate", "pa_kv_cache_num_blocks", "pa_kv_cache_get",
     "pa_kv_cache_copy_blocks", "pa_normalize_num_kv_blocks", "pa_evictor_create", "pa_score_manager_create",
@@ -97,6 +98,7 @@ def lib():
         "pa_forward": (i32, [vp, i32, P(pa_layer_io)]),
         "pa_kv_append": (i32, [vp, i32, P(pa_layer_io)]),
         "pa_attention": (i32, [vp, i32, P(pa_layer_io)]),
+        "pa_attention_static": (i32, [vp, i32, P(pa_layer_io)]),
         "pa_synchronize": (i32, [vp]),
         "pa_get_num_splits": (i32, [vp]),
         "pa_set_profiling": (i32, [vp, i32]),

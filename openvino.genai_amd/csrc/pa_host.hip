@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -71,12 +72,36 @@ void check_config(const pa_config* c) {
     PA_REQUIRE(c->device >= 0 && c->device < ndev, PA_OUT_OF_BOUNDS, "no such HIP device");
 }
 
+// Fixed device scratch of pa_attention_static: one copy per GPU the library runs on, held until the process ends.
+// In host code this name is only a handle for hipGetSymbolAddress; device code and every launch use the resolved
+// pointer.
+constexpr size_t STATIC_SCRATCH_BYTES = PA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// The device address of `scratch` on `device`, which must be the current device.
+void* resolve_static_scratch(int device) {
+    PA_REQUIRE(device >= 0 && device < MAX_DEVICES, PA_OUT_OF_BOUNDS, "device ordinal beyond the scratch table");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        PA_REQUIRE(p, PA_GENERAL_ERROR, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[device] = p;
+    }
+    return g_scratch_ptr[device];
+}
+
 }  // namespace
 
 struct pa_ctx {
     pa_config cfg{};
     hipStream_t stream = nullptr;
     std::string error;
+    uint8_t* static_scratch = nullptr;  // this device's copy of the fixed scratch (pa_attention_static)
     // step state
     bool step_ready = false;
     int32_t B = 0, T = 0, max_kv = 0, total_scores = 0, total_block_ids = 0, nsplit = 1, generic_nsplit = 1;
@@ -397,7 +422,58 @@ void plan_items(pa_ctx* ctx) {
     ctx->tok_nsplit_off = item_bytes;
 }
 
-void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
+// Workspace of a decode launch (split partials, final maxima and denominators, per-kv-head score sums or per-head
+// split probabilities): the context's growable buffers, or -- from_static -- pieces of the fixed device scratch, in
+// which case nothing is allocated and a step that needs more than the scratch holds is refused.
+struct DecodeWs {
+    float *part_acc, *part_ml, *final_ml, *group_scores;
+    _Float16* p_split;
+};
+
+DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_scores, bool from_static) {
+    const pa_config& c = ctx->cfg;
+    const size_t b_final = rows * 2 * sizeof(float);
+    const size_t b_acc = nsplit > 1 ? rows * nsplit * c.head_size * sizeof(float) : 0;
+    const size_t b_ml = nsplit > 1 ? rows * nsplit * 2 * sizeof(float) : 0;
+    const size_t b_group = want_scores && nsplit == 1 ? (size_t)c.num_kv_heads * ctx->total_scores * sizeof(float) : 0;
+    const size_t b_psplit = want_scores && nsplit > 1
+                                ? (size_t)c.num_heads * pa::p_split_stride(ctx->total_scores, ctx->B) * sizeof(uint16_t) : 0;
+    DecodeWs w{};
+    if (from_static) {
+        size_t off = 0;
+        auto place = [&](size_t bytes) {
+            const size_t at = off;
+            off += (bytes + 255) & ~(size_t)255;
+            return at;
+        };
+        const size_t o_final = place(b_final), o_acc = place(b_acc), o_ml = place(b_ml), o_group = place(b_group),
+                     o_psplit = place(b_psplit);
+        PA_REQUIRE(off <= STATIC_SCRATCH_BYTES, PA_OUT_OF_BOUNDS,
+                   "pa_attention_static: this step needs " + std::to_string(off) + " bytes of workspace, the fixed scratch holds " +
+                       std::to_string(STATIC_SCRATCH_BYTES) + " (use pa_attention)");
+        PA_REQUIRE(ctx->static_scratch, PA_NOT_ALLOCATED, "the fixed scratch of this device was not resolved");
+        uint8_t* base = ctx->static_scratch;
+        w.final_ml = reinterpret_cast<float*>(base + o_final);
+        w.part_acc = reinterpret_cast<float*>(base + o_acc);
+        w.part_ml = reinterpret_cast<float*>(base + o_ml);
+        w.group_scores = reinterpret_cast<float*>(base + o_group);
+        w.p_split = reinterpret_cast<_Float16*>(base + o_psplit);
+        return w;
+    }
+    ctx->final_ml.reserve(b_final);
+    if (b_acc) ctx->part_acc.reserve(b_acc);
+    if (b_ml) ctx->part_ml.reserve(b_ml);
+    if (b_group) ctx->group_scores.reserve(b_group);
+    if (b_psplit) ctx->p_split.reserve(b_psplit);
+    w.final_ml = ctx->final_ml.as<float>();
+    w.part_acc = ctx->part_acc.as<float>();
+    w.part_ml = ctx->part_ml.as<float>();
+    w.group_scores = ctx->group_scores.as<float>();
+    w.p_split = ctx->p_split.as<_Float16>();
+    return w;
+}
+
+void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static_ws = false) {
     check_io(ctx, io, false, true);
     const int32_t* table = table_for(ctx, layer);
     const pa_config& c = ctx->cfg;
@@ -410,6 +486,11 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
     const bool use_decode16 = use_mfma && decode16_shape(c) && !ctx->h_dec16.empty() &&
                               ctx->n_single + ctx->n_sparse == ctx->n_items;
     const bool mfma_left = use_mfma && !(use_decode16 && ctx->n_single == ctx->n_items);
+    if (static_ws)
+        PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
+                   PA_NOT_IMPLEMENTED,
+                   "pa_attention_static serves steps in which every sequence schedules one token, over a u8 cache or a "
+                   "16-bit cache of the query's type (block size 32, head size 64 or 128, at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
     if (use_decode) {
@@ -423,27 +504,17 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
         a.n_seqs = (int32_t)ctx->h_dec.size();
         a.seq_list = a.n_seqs == ctx->B ? nullptr : ctx->dec_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
-        ctx->final_ml.reserve(rows * 2 * sizeof(float));
-        if (a.nsplit > 1) {
-            ctx->part_acc.reserve(rows * a.nsplit * c.head_size * sizeof(float));
-            ctx->part_ml.reserve(rows * a.nsplit * 2 * sizeof(float));
-        }
-        if (io->scores) {
-            if (a.nsplit == 1)
-                ctx->group_scores.reserve((size_t)c.num_kv_heads * ctx->total_scores * sizeof(float));
-            else
-                ctx->p_split.reserve((size_t)c.num_heads * pa::p_split_stride(ctx->total_scores, ctx->B) * sizeof(uint16_t));
-        }
+        const DecodeWs ws = decode_workspace(ctx, rows, a.nsplit, io->scores != nullptr, static_ws);
         a.query = static_cast<const uint16_t*>(io->query);
         a.key_cache = static_cast<const uint8_t*>(io->key_cache);
         a.value_cache = static_cast<const uint8_t*>(io->value_cache);
         a.block_indices = table;
         a.out = static_cast<uint16_t*>(io->out);
-        a.part_acc = ctx->part_acc.as<float>();
-        a.part_ml = ctx->part_ml.as<float>();
-        a.final_ml = ctx->final_ml.as<float>();
-        a.group_scores = ctx->group_scores.as<float>();
-        a.p_split = ctx->p_split.as<_Float16>();
+        a.part_acc = ws.part_acc;
+        a.part_ml = ws.part_ml;
+        a.final_ml = ws.final_ml;
+        a.group_scores = ws.group_scores;
+        a.p_split = ws.p_split;
         HIP_CHECK(pa::launch_decode_u8(ctx->stream, a, c.query_dtype, io->scores, ctx->max_kv,
                                        use_mfma ? nullptr : ev0, use_mfma ? nullptr : ev1));
         ctx->timed = ctx->profiling;
@@ -460,27 +531,17 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
         a.n_seqs = (int32_t)ctx->h_dec16.size();
         a.seq_list = a.n_seqs == ctx->B ? nullptr : ctx->dec16_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
-        ctx->final_ml.reserve(rows * 2 * sizeof(float));
-        if (a.nsplit > 1) {
-            ctx->part_acc.reserve(rows * a.nsplit * c.head_size * sizeof(float));
-            ctx->part_ml.reserve(rows * a.nsplit * 2 * sizeof(float));
-        }
+        const DecodeWs ws = decode_workspace(ctx, rows, a.nsplit, io->scores != nullptr, static_ws);
         a.query = static_cast<const uint16_t*>(io->query);
         a.key_cache = static_cast<const uint8_t*>(io->key_cache);
         a.value_cache = static_cast<const uint8_t*>(io->value_cache);
         a.block_indices = table;
         a.out = static_cast<uint16_t*>(io->out);
-        a.part_acc = ctx->part_acc.as<float>();
-        a.part_ml = ctx->part_ml.as<float>();
-        a.final_ml = ctx->final_ml.as<float>();
-        if (io->scores) {
-            if (a.nsplit == 1)
-                ctx->group_scores.reserve((size_t)c.num_kv_heads * ctx->total_scores * sizeof(float));
-            else
-                ctx->p_split.reserve((size_t)c.num_heads * pa::p_split_stride(ctx->total_scores, ctx->B) * sizeof(uint16_t));
-        }
-        a.group_scores = ctx->group_scores.as<float>();
-        a.p_split = ctx->p_split.as<_Float16>();
+        a.part_acc = ws.part_acc;
+        a.part_ml = ws.part_ml;
+        a.final_ml = ws.final_ml;
+        a.group_scores = ws.group_scores;
+        a.p_split = ws.p_split;
         HIP_CHECK(pa::launch_decode16(ctx->stream, a, c.query_dtype, io->scores, ctx->max_kv, mfma_left ? nullptr : ev0,
                                       mfma_left ? nullptr : ev1));
         ctx->timed = ctx->profiling;
@@ -580,9 +641,11 @@ int32_t pa_create(const pa_config* cfg, pa_ctx** out) {
         *out = nullptr;
         check_config(cfg);
         HIP_CHECK(hipSetDevice(cfg->device));
+        uint8_t* fixed = static_cast<uint8_t*>(resolve_static_scratch(cfg->device));
         pa_ctx* ctx = new pa_ctx();
         ctx->cfg = *cfg;
         ctx->stream = static_cast<hipStream_t>(cfg->stream);
+        ctx->static_scratch = fixed;
         *out = ctx;
     });
 }
@@ -917,6 +980,14 @@ int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
     return guarded(ctx, [&] {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         do_attention(ctx, layer, io);
+    });
+}
+
+int32_t pa_attention_static(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
+    if (!ctx) return PA_INVALID_C_PARAM;
+    return guarded(ctx, [&] {
+        HIP_CHECK(hipSetDevice(ctx->cfg.device));
+        do_attention(ctx, layer, io, true);
     });
 }
 

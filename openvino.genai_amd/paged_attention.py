@@ -85,6 +85,12 @@ class PagedAttention:
         io = self._io(query, None, None, key_cache, value_cache, out, scores)
         self._ck(L.lib().pa_attention(self._h, layer, C.byref(io)))
 
+    def attention_static(self, query, key_cache, value_cache, out, scores=None, layer=0):
+        """``attention`` without any allocation inside the call: workspaces come from the library's fixed device
+        scratch (single-token steps only; a step that needs more than the scratch holds raises OUT_OF_BOUNDS)."""
+        io = self._io(query, None, None, key_cache, value_cache, out, scores)
+        self._ck(L.lib().pa_attention_static(self._h, layer, C.byref(io)))
+
     def forward(self, query, key, value, key_cache, value_cache, out, scores=None, layer=0):
         io = self._io(query, key, value, key_cache, value_cache, out, scores)
         self._ck(L.lib().pa_forward(self._h, layer, C.byref(io)))

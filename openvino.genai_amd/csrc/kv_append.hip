@@ -19,7 +19,6 @@ __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, co
                                                         uint8_t* __restrict__ key_cache,
                                                         uint8_t* __restrict__ value_cache,
                                                         const int32_t* __restrict__ block_indices) {
-#pragma clang fp contract(off)
     const int lane = threadIdx.x & 63;
     const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     const long rows = (long)st.T * sh.Hkv * 2;
@@ -36,42 +35,10 @@ __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, co
     uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)rb;
 
     uint16_t raw[EPL];
-    if constexpr (EPL == 4) {
-        uint2 v = *reinterpret_cast<const uint2*>(src);
-        raw[0] = v.x & 0xffff; raw[1] = v.x >> 16; raw[2] = v.y & 0xffff; raw[3] = v.y >> 16;
-    } else if constexpr (EPL == 2) {
-        uint32_t v = *reinterpret_cast<const uint32_t*>(src);
-        raw[0] = v & 0xffff; raw[1] = v >> 16;
-    } else {
-        raw[0] = src[0];
-    }
+    load_row16<EPL>(src, raw);
 
     if (KVDT == DT_U8) {
-        float x[EPL];
-        float mn, mx;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) x[e] = load16<QDT>(raw[e]);
-        mn = mx = x[0];
-#pragma unroll
-        for (int e = 1; e < EPL; ++e) { mn = fminf(mn, x[e]); mx = fmaxf(mx, x[e]); }
-        mn = wave_min(mn);
-        mx = wave_max(mx);
-        float scale = (mx - mn) / 255.0f;
-        if (scale == 0.0f) scale = 0.0001f;
-        const float zp = -mn / scale;
-        const float inv = 1.0f / scale;
-        uint32_t packed = 0;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            float v = rintf(__fmaf_rn(x[e], inv, zp));
-            v = fminf(fmaxf(v, 0.0f), 255.0f);
-            packed |= (uint32_t)(int)v << (8 * e);
-        }
-        if (lane == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
-        uint8_t* c = dst + 8 + lane * EPL;
-        if constexpr (EPL == 4) *reinterpret_cast<uint32_t*>(c) = packed;
-        else if constexpr (EPL == 2) *reinterpret_cast<uint16_t*>(c) = (uint16_t)packed;
-        else *c = (uint8_t)packed;
+        quantize_row_u8<QDT, EPL>(raw, dst, lane);
     } else {
         uint16_t o[EPL];
 #pragma unroll

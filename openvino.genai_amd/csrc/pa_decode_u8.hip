@@ -20,6 +20,8 @@
 // are known they are normalised, summed over the group's heads and written out.
 //
 // Roofline: HBM.  Algorithmic bytes per (sequence, kv head, position): 2 * (D + 8).
+#include <type_traits>
+
 #include "pa_device.h"
 
 namespace pa {
@@ -91,37 +93,60 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     constexpr int KS = D / 32;             // k-steps of the QK contraction
     constexpr int RT = D / 16;             // 16-row output tiles of PV
     constexpr int VB = D / 16;             // V bytes per lane per token row
+    constexpr int SLOT = TILE;             // a wave's LDS staging slot: a K block, then a V block
+    constexpr int EPL = D / 64;            // elements per lane of a new K / V row
     static_assert(TILE == FULL * 1024 + 256, "tile = whole passes + 16 chunks");
     extern __shared__ __align__(16) uint8_t smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, g = lane >> 4;
     const StepDev& st = a.st;
     const int Hq = a.sh.Hq, Hkv = a.sh.Hkv, G = a.G, nsplit = a.nsplit;
 
-    const int split = blockIdx.x % nsplit;
-    const int hkv = (blockIdx.x / nsplit) % Hkv;
-    const int b = a.seq_list ? a.seq_list[blockIdx.x / (nsplit * Hkv)] : (int)(blockIdx.x / (nsplit * Hkv));
-    const int t = st.subsequence_begins[b];
-    const int kv_len = st.past_lens[b] + 1;
-    const int first = st.sliding_window > 0 ? max(0, kv_len - st.sliding_window) : 0;
-    const int tile_lo = first / TOK, tile_hi = (kv_len + TOK - 1) / TOK;
-    const int per = ceil_div(tile_hi - tile_lo, nsplit);
-    const int tb = tile_lo + split * per;
-    const int te = min(tile_hi, tb + per);
-    const int32_t* table = a.block_indices + st.block_indices_begins[b];
+    // grid = (split, kv head, listed sequence)
+    const int split = blockIdx.x, hkv = blockIdx.y;
+    // everything the first block fetches depend on sits in one descriptor (one scalar load)
+    const DecodeDesc* __restrict__ dsc = a.descs + ((long)blockIdx.z * nsplit + split);
+    const int b = dsc->b, t = dsc->t, kv_len = dsc->kv_len, first = dsc->first;
+    const int tb = dsc->tb, te = dsc->te;
+    const int tile_hi = (kv_len + TOK - 1) / TOK;
+    const int32_t* table = a.block_indices + dsc->table_off;
 
     // LDS carve-up
-    uint8_t* slot = smem + wv * TILE;                                  // wave-private staging
-    float* wave_mlz = reinterpret_cast<float*>(smem + WAVES * TILE);   // [WAVES][16][4]
+    uint8_t* slot = smem + wv * SLOT;                                  // wave-private staging
+    float* wave_mlz = reinterpret_cast<float*>(smem + WAVES * SLOT);   // [WAVES][16][4]
     float* msnap = wave_mlz + WAVES * 16 * 4;                          // [max_tiles][16]
     _Float16* ptile = reinterpret_cast<_Float16*>(msnap + (a.want_scores ? a.max_tiles * 16 : 0));  // [G][max_tiles*TOK]
     const int pstride = a.max_tiles * TOK;
-    // the first block's loads go out before anything else is fetched
+
+    // The step's new K / V row of this (sequence, kv head) goes into the caches here when the step's append is fused
+    // into this launch: by the wave that later reads the sequence's last block.  That wave's loads of the block must
+    // see the row: with few blocks ahead of it the wave waits for the stores before it fetches anything; otherwise the
+    // stores follow its first fetches, and at least two of its blocks -- each consumed behind a wait that covers
+    // everything issued before it -- lie between the stores and the fetch of the last block.
+    const bool appends = a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
+    const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
+    auto append_rows = [&]() __attribute__((always_inline)) {
+        const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
+        const long dst = (((long)dsc->last_id * Hkv + hkv) * TOK + (kv_len - 1) % TOK) * ROW;
+        uint16_t kr[EPL], vr[EPL];
+        load_row16<EPL>(a.key + src, kr);
+        load_row16<EPL>(a.value + src, vr);
+        quantize_row_u8<QDT, EPL>(kr, const_cast<uint8_t*>(a.key_cache) + dst, lane);
+        quantize_row_u8<QDT, EPL>(vr, const_cast<uint8_t*>(a.value_cache) + dst, lane);
+    };
+    if (append_first) {
+        append_rows();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+
+    // the first two blocks' loads go out before anything else is fetched
     u4v kraw[FULL], vraw[FULL], traw, kraw2[FULL], vraw2[FULL], traw2;
     int tile = tb + wv;
-    if (tile < te) issue_block<FULL>(a, table[tile], hkv, TILE, lane, kraw, vraw, traw);
-    if (tile + WAVES < te) issue_block<FULL>(a, table[tile + WAVES], hkv, TILE, lane, kraw2, vraw2, traw2);
+    if (tile < te) issue_block<FULL>(a, dsc->ids[wv], hkv, TILE, lane, kraw, vraw, traw);
+    if (tile + WAVES < te) issue_block<FULL>(a, dsc->ids[wv + WAVES], hkv, TILE, lane, kraw2, vraw2, traw2);
+    if (appends && !append_first) append_rows();
     // this workgroup's slice of the block table, so that no later block fetch waits on a table fetch
     int32_t* tab = reinterpret_cast<int32_t*>(smem + a.table_off);
     for (int i = tid; i < te - tb; i += NT) tab[i] = table[tb + i];
@@ -154,7 +179,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
         }
         qsum = xor_reduce_sum_g(qsum);
     }
-    const float scl = st.scale * LOG2E;  // logits are kept in the log2 domain
+    const float scl24 = st.scale * LOG2E * TWO24;  // logits are kept in the log2 domain
+    const float qsum24 = qsum * (1.0f / TWO24);
 
     float m_run = -INFINITY, l_part = 0.0f, z_part = 0.0f;
     f4 acc[RT];
@@ -201,69 +227,76 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
         __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax (log2 domain) -------------------------------------------------------
-        float x[8];
-        bool seen[8];  // rows outside [first, kv_len) may hold anything, headers included
-        float mx = -INFINITY;
-        const int pos0 = tile * TOK;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float raw = (j < 4) ? sc0[j & 3] : sc1[j & 3];
-            const float fk = hk[j].x * scl;
-            const int pos = pos0 + 16 * (j >> 2) + 4 * g + (j & 3);
-            float v = raw * (TWO24 * fk) - hk[j].y * qsum * fk;
-            seen[j] = pos < kv_len && pos >= first;
-            v = seen[j] ? v : -INFINITY;
-            x[j] = v;
-            mx = fmaxf(mx, v);
-        }
-        mx = xor_reduce_max_g(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
-        float2 hv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            hv[j] = *reinterpret_cast<const float2*>(slot + ROW * (16 * (j >> 2) + 4 * g + (j & 3)));
-        float psum = 0.0f, zsum = 0.0f;
+        // Rows outside [first, kv_len) may hold anything, headers included: blocks that reach beyond either end
+        // mask them (EDGE); the blocks in between, nearly all of a long context, skip the tests and selects.
         h8 pb, pl;
-        _Float16 ph[8];
-        float wf[8];
+        auto softmax = [&](auto edge_tag) __attribute__((always_inline)) {
+            constexpr bool EDGE = decltype(edge_tag)::value;
+            float x[8];
+            bool seen[8];
+            float mx = -INFINITY;
+            const int pos0 = tile * TOK;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float p = __builtin_amdgcn_exp2f(x[j] - m_new);
-            wf[j] = seen[j] ? p * hv[j].x : 0.0f;
-            psum += p;
-            pb[j] = (_Float16)wf[j];
-            ph[j] = (_Float16)p;
-        }
-        // the zero-point term must see the same rounded weight as the matrix product, or the rounding error is scaled
-        // by the code instead of by (code - zp).  The weights are pinned in their registers first: the compiler may
-        // otherwise form the f16 value twice (from the f32 product, and with a mixed-precision multiply), and the two
-        // differ by one f16 step at a tie
-        asm volatile("" : "+v"(pb));
-        // what the rounding to f16 dropped goes through the matrix pipe as a second operand: with 11 bits alone a
-        // row that leans on a few tokens with large V values of opposite sign can miss the tolerance
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pl[j] = (_Float16)(wf[j] - (float)pb[j]);
-        asm volatile("" : "+v"(pl));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) zsum += seen[j] ? ((float)pb[j] + (float)pl[j]) * hv[j].y : 0.0f;
-        l_part = l_part * corr + psum;
-        z_part = z_part * corr + zsum;
-        m_run = m_new;
-        if (__any(corr != 1.0f)) {
-#pragma unroll
-            for (int r = 0; r < RT; ++r) acc[r] *= corr;
-        }
-        if (a.want_scores) {
-            const int lt = tile - tb;
-            if (n < G) {
-                _Float16* dst = ptile + n * pstride + lt * TOK + 4 * g;
-                typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-                *reinterpret_cast<h4*>(dst) = h4{ph[0], ph[1], ph[2], ph[3]};
-                *reinterpret_cast<h4*>(dst + 16) = h4{ph[4], ph[5], ph[6], ph[7]};
-                if (g == 0) msnap[lt * 16 + n] = m_new;
+            for (int j = 0; j < 8; ++j) {
+                const float raw = (j < 4) ? sc0[j & 3] : sc1[j & 3];
+                const int pos = pos0 + 16 * (j >> 2) + 4 * g + (j & 3);
+                // scale * sc_k * (q . codes - zp_k * sum(q)), the code products still carrying their 2^-24
+                float v = (hk[j].x * scl24) * __builtin_fmaf(-hk[j].y, qsum24, raw);
+                seen[j] = !EDGE || (pos < kv_len && pos >= first);
+                v = seen[j] ? v : -INFINITY;
+                x[j] = v;
+                mx = fmaxf(mx, v);
             }
-        }
+            mx = xor_reduce_max_g(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+            float2 hv[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                hv[j] = *reinterpret_cast<const float2*>(slot + ROW * (16 * (j >> 2) + 4 * g + (j & 3)));
+            float psum = 0.0f, zsum = 0.0f;
+            _Float16 ph[8];
+            float wf[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float p = __builtin_amdgcn_exp2f(x[j] - m_new);
+                wf[j] = seen[j] ? p * hv[j].x : 0.0f;
+                psum += p;
+                pb[j] = (_Float16)wf[j];
+                ph[j] = (_Float16)p;
+            }
+            // The weights are pinned in their registers: the compiler may otherwise form the f16 value twice (from the
+            // f32 product, and with a mixed-precision multiply), and the two differ by one f16 step at a tie
+            asm volatile("" : "+v"(pb));
+            // what the rounding to f16 dropped goes through the matrix pipe as a second operand: with 11 bits alone a
+            // row that leans on a few tokens with large V values of opposite sign can miss the tolerance
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pl[j] = (_Float16)(wf[j] - (float)pb[j]);
+            asm volatile("" : "+v"(pl));
+            // the zero-point term must see the weight the matrix product sees, or the rounding error is scaled by the
+            // code instead of by (code - zp); the two halves together carry it to 2^-22, so the f32 weight serves
+#pragma unroll
+            for (int j = 0; j < 8; ++j) zsum += seen[j] ? wf[j] * hv[j].y : 0.0f;
+            l_part = l_part * corr + psum;
+            z_part = z_part * corr + zsum;
+            m_run = m_new;
+            if (__any(corr != 1.0f)) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r) acc[r] *= corr;
+            }
+            if (a.want_scores) {
+                const int lt = tile - tb;
+                if (n < G) {
+                    _Float16* dst = ptile + n * pstride + lt * TOK + 4 * g;
+                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                    *reinterpret_cast<h4*>(dst) = h4{ph[0], ph[1], ph[2], ph[3]};
+                    *reinterpret_cast<h4*>(dst + 16) = h4{ph[4], ph[5], ph[6], ph[7]};
+                    if (g == 0) msnap[lt * 16 + n] = m_new;
+                }
+            }
+        };
+        if (tile * TOK < first || tile * TOK + TOK > kv_len) softmax(std::true_type{});
+        else softmax(std::false_type{});
 
         // ---- O^T[d][head] += V^T . P^T ----------------------------------------------------------
         // lane (m = n, g) reads its VB bytes d = VB*m .. of each of its eight token rows
@@ -298,6 +331,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     }
 
     // ---- merge the waves ---------------------------------------------------------------------------
+    // Every wave leaves (max, denominator, zero-point sum) per head and its raw accumulators of the group's heads
+    // (lanes n < G) in LDS; after one barrier each thread folds the waves for two channels of one head.
     const float l_w = xor_reduce_sum_g(l_part);
     const float z_w = xor_reduce_sum_g(z_part);
     __syncthreads();  // staging slots are dead from here on
@@ -306,77 +341,83 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
         wave_mlz[(wv * 16 + n) * 4 + 1] = l_w;
         wave_mlz[(wv * 16 + n) * 4 + 2] = z_w;
     }
-    __syncthreads();
-    float M = -INFINITY;
+    // folds the waves' (m, l, z) of one head: the maximum, each wave's factor, denominator and zero-point sum
+    auto fold_head = [&](const int head, float (&f)[WAVES], float& M, float& L, float& Z) __attribute__((always_inline)) {
+        M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) M = fmaxf(M, wave_mlz[(w * 16 + n) * 4]);
-    float L = 0.0f, Z = 0.0f;
+        for (int w = 0; w < WAVES; ++w) M = fmaxf(M, wave_mlz[(w * 16 + head) * 4]);
+        L = 0.0f;
+        Z = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-        const float mw = wave_mlz[(w * 16 + n) * 4];
-        const float f = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
-        L += wave_mlz[(w * 16 + n) * 4 + 1] * f;
-        Z += wave_mlz[(w * 16 + n) * 4 + 2] * f;
-    }
-    const float f_own = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
-    // accumulators: [WAVES][RT*4][64] floats in the dead staging area, half of the tiles at a time
+        for (int w = 0; w < WAVES; ++w) {
+            const float mw = wave_mlz[(w * 16 + head) * 4];
+            f[w] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
+            L += wave_mlz[(w * 16 + head) * 4 + 1] * f[w];
+            Z += wave_mlz[(w * 16 + head) * 4 + 2] * f[w];
+        }
+    };
+    // accumulators: [WAVES][HC][D] floats in the dead staging area, HC heads at a time
+    constexpr int HC = 8;
+    static_assert((size_t)WAVES * HC * D * sizeof(float) <= (size_t)WAVES * SLOT, "accumulators of a pass fit the staging area");
     float* red = reinterpret_cast<float*>(smem);
-    constexpr int HALF = RT / 2;
     const bool final_out = nsplit == 1;
-    const int hq = hkv * G + n;
-    const long prow = ((long)t * Hq + hq) * nsplit + split;
-    const float inv_l = L > 0.0f ? 1.0f / L : 0.0f;
-    if (a.want_scores) {
-        // one factor per (block, head): exp2(snapshot - M) (/ L when this workgroup saw the whole context), written
-        // over the snapshot.  Entry e belongs to head e % 16 = this thread's n; the barrier inside the merge below
-        // publishes the factors
-        const float fl = final_out ? inv_l : 1.0f;
-        for (int e = tid; e < max(te - tb, 0) * 16; e += 64 * WAVES)
-            msnap[e] = n < G ? __builtin_amdgcn_exp2f(msnap[e] - M) * fl : 0.0f;
-    }
+    for (int n0 = 0; n0 < G; n0 += HC) {
+        if (n0) __syncthreads();
+        if (n >= n0 && n < min(G, n0 + HC)) {
+            float* dst = red + ((wv * HC + n - n0) * D) + (D / 4) * g;
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        if (half) __syncthreads();
+            for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int r = 0; r < HALF; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) red[(wv * HALF * 4 + r * 4 + i) * 64 + lane] = acc[half * HALF + r][i] * f_own;
+                for (int i = 0; i < 4; ++i) dst[VB * i + r] = acc[r][i];  // lane (n, g), register i of tile r: d = (D/4) g + VB i + r
+        }
         __syncthreads();
-        // wave w finishes tile r = w of this half (HALF == WAVES for D = 128; HALF = 2 for D = 64)
-        for (int r = wv; r < HALF; r += WAVES) {
-            const int rr = half * HALF + r;
+        if (n0 == 0 && a.want_scores) {
+            // one factor per (block, head): exp2(snapshot - M) (/ L when this workgroup saw the whole context), written
+            // over the snapshot.  Entry e belongs to head e % 16 = this thread's n; the barrier before the score
+            // phase publishes the factors
+            float f[WAVES], M, L, Z;
+            fold_head(n, f, M, L, Z);
+            const float fl = final_out ? (L > 0.0f ? 1.0f / L : 0.0f) : 1.0f;
+            for (int e = tid; e < max(te - tb, 0) * 16; e += NT)
+                msnap[e] = n < G ? __builtin_amdgcn_exp2f(msnap[e] - M) * fl : 0.0f;
+        }
+        const int heads = min(G, n0 + HC) - n0;
+        for (int idx = tid; idx < heads * (D / 2); idx += NT) {
+            const int hl = idx / (D / 2), d = 2 * (idx % (D / 2));
+            const int head = n0 + hl, hq = hkv * G + head;
+            float f[WAVES], M, L, Z;
+            fold_head(head, f, M, L, Z);
+            float v0 = 0.0f, v1 = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v = 0.0f;
-#pragma unroll
-                for (int w = 0; w < WAVES; ++w) v += red[(w * HALF * 4 + r * 4 + i) * 64 + lane];
-                // lane (n, g), register i of tile rr holds d = (D/4) g + VB i + rr of head n
-                const int d = (D / 4) * g + VB * i + rr;
-                const float o = v * TWO24 - Z;
-                if (n < G) {
-                    if (final_out) a.out[((long)t * Hq + hq) * D + d] = store16<QDT>(o * inv_l);
-                    else a.part_acc[prow * D + d] = o;
-                }
+            for (int w = 0; w < WAVES; ++w) {
+                const float2 v = *reinterpret_cast<const float2*>(red + (w * HC + hl) * D + d);
+                v0 += v.x * f[w];
+                v1 += v.y * f[w];
+            }
+            const float o0 = v0 * TWO24 - Z, o1 = v1 * TWO24 - Z;
+            const long prow = ((long)t * Hq + hq) * nsplit + split;
+            if (final_out) {
+                const float inv_l = L > 0.0f ? 1.0f / L : 0.0f;
+                *reinterpret_cast<uint32_t*>(a.out + ((long)t * Hq + hq) * D + d) =
+                    (uint32_t)store16<QDT>(o0 * inv_l) | ((uint32_t)store16<QDT>(o1 * inv_l) << 16);
+            } else {
+                *reinterpret_cast<float2*>(a.part_acc + prow * D + d) = make_float2(o0, o1);
+            }
+            if (d == 0) {  // maxima stay in the log2 domain within this kernel family
+                float* ml = final_out ? a.final_ml + 2 * ((long)t * Hq + hq) : a.part_ml + 2 * prow;
+                ml[0] = M;
+                ml[1] = L;
             }
         }
     }
-    if (wv == 0 && g == 0 && n < G) {
-        // maxima stay in the log2 domain within this kernel family
-        if (final_out) {
-            a.final_ml[2 * ((long)t * Hq + hq)] = M;
-            a.final_ml[2 * ((long)t * Hq + hq) + 1] = L;
-        } else {
-            a.part_ml[2 * prow] = M;
-            a.part_ml[2 * prow + 1] = L;
-        }
-    }
 
-    // ---- scores: the factors were formed in place of the block maxima before the merge --------------
+    // ---- scores: the factors were formed in place of the block maxima during the merge ---------------
     if (!a.want_scores) return;
+    __syncthreads();
     const float* fac = msnap;
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
     typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-    const long soff = st.score_offsets[b];
+    const long soff = dsc->score_off;
     if (final_out) {
         // sum over the group's heads -> group_scores[hkv][position], four positions per thread;
         // positions before the first block of the window get 0
@@ -603,9 +644,9 @@ static hipError_t launch_decode_typed(hipStream_t s, const DecodeArgs& a_in, flo
     auto kern = pa_decode_u8_kernel<D, QDT, WAVES>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    const unsigned wgs = (unsigned)a.n_seqs * a.sh.Hkv * a.nsplit;
+    if (a.n_seqs > 65535) return hipErrorInvalidValue;  // grid z
     if (ev0) (void)hipEventRecord(ev0, s);
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * WAVES), lds, s, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)a.nsplit, (unsigned)a.sh.Hkv, (unsigned)a.n_seqs), dim3(64 * WAVES), lds, s, a);
     if (ev1) (void)hipEventRecord(ev1, s);
     return launch_decode_post(s, a, QDT, scores, max_kv_len);
 }

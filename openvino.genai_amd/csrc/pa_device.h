@@ -55,6 +55,54 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
+// ---- one K or V row into a u8 cache row ---------------------------------------------------------
+// A 64-lane wave quantises one row of D = 64 * EPL elements: `f32 scale | f32 zero-point | D codes` with
+//   scale = (max - min) / 255  (a zero range takes 1e-4),  zp = -min / scale,
+//   code  = clamp(rne(fma(x, 1/scale, zp)), 0, 255),
+// every operation in IEEE binary32 (no contraction), so that the bytes are reproducible on any IEEE host.
+// `raw` holds the lane's EPL consecutive elements (bit patterns of QDT); `dst` is the row's first byte.
+template <int QDT, int EPL>
+__device__ __forceinline__ void quantize_row_u8(const uint16_t (&raw)[EPL], uint8_t* dst, const int lane) {
+#pragma clang fp contract(off)
+    float x[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) x[e] = load16<QDT>(raw[e]);
+    float mn = x[0], mx = x[0];
+#pragma unroll
+    for (int e = 1; e < EPL; ++e) { mn = fminf(mn, x[e]); mx = fmaxf(mx, x[e]); }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    float scale = (mx - mn) / 255.0f;
+    if (scale == 0.0f) scale = 0.0001f;
+    const float zp = -mn / scale;
+    const float inv = 1.0f / scale;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        float v = rintf(__fmaf_rn(x[e], inv, zp));
+        v = fminf(fmaxf(v, 0.0f), 255.0f);
+        packed |= (uint32_t)(int)v << (8 * e);
+    }
+    if (lane == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
+    uint8_t* c = dst + 8 + lane * EPL;
+    if constexpr (EPL == 4) *reinterpret_cast<uint32_t*>(c) = packed;
+    else if constexpr (EPL == 2) *reinterpret_cast<uint16_t*>(c) = (uint16_t)packed;
+    else *c = (uint8_t)packed;
+}
+// The lane's EPL consecutive elements of a row of 16-bit values.
+template <int EPL>
+__device__ __forceinline__ void load_row16(const uint16_t* src, uint16_t (&raw)[EPL]) {
+    if constexpr (EPL == 4) {
+        const uint2 v = *reinterpret_cast<const uint2*>(src);
+        raw[0] = v.x & 0xffff; raw[1] = v.x >> 16; raw[2] = v.y & 0xffff; raw[3] = v.y >> 16;
+    } else if constexpr (EPL == 2) {
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(src);
+        raw[0] = v & 0xffff; raw[1] = v >> 16;
+    } else {
+        raw[0] = src[0];
+    }
+}
+
 // ---- step metadata as the kernels see it (all device pointers) --------------------------------
 struct StepDev {
     const int32_t* past_lens;             // [B]
@@ -92,6 +140,21 @@ hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const Shap
                                     const int32_t* block_indices, const AttnWorkspace& ws, void* out, float* scores,
                                     int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1);
 
+// What a workgroup of the u8 decode kernel needs to start fetching KV blocks, resolved on the host when the block
+// table is set: one entry per (listed sequence, split), read with one scalar load instead of a chain of dependent
+// loads through the step arrays and the table.
+struct DecodeDesc {
+    int32_t b, t;           // sequence and its token row
+    int32_t kv_len, first;  // context length (new token included) and first visible position
+    int32_t tb, te;         // KV blocks [tb, te) of this split
+    int32_t table_off;      // first entry of the sequence's block table
+    int32_t score_off;      // first entry of the sequence in `scores`
+    int32_t last_id;        // physical id of the block that holds position kv_len - 1
+    int32_t pad[7];
+    int32_t ids[16];        // physical ids of the split's first 16 blocks (0 beyond te)
+};
+static_assert(sizeof(DecodeDesc) == 128, "one descriptor = 128 bytes");
+
 // Arguments of the u8 decode kernel family (pa_decode_u8.hip).
 struct DecodeArgs {
     StepDev st;
@@ -101,6 +164,10 @@ struct DecodeArgs {
     const uint8_t* value_cache;
     const int32_t* block_indices;
     const int32_t* seq_list;      // sequences this launch covers (single-token ones); null = all B
+    const DecodeDesc* descs;      // u8 kernel: [n_seqs][nsplit]
+    const uint16_t* key;          // u8 kernel with fuse_append: the step's new K / V rows [T, Hkv*D], which the
+    const uint16_t* value;        // workgroup that owns a sequence's last block quantises into the caches itself
+    int32_t fuse_append;
     int32_t n_seqs;
     int32_t G;                    // query heads per kv head (<= 16)
     int32_t nsplit;               // workgroups per (sequence, kv head)

@@ -139,6 +139,12 @@ struct pa_ctx {
     // block tables: shared (index 0 of `tables` when shared) or per layer
     std::vector<DevBuf> tables;
     std::vector<int32_t> table_count;
+    std::vector<int64_t> table_bound;  // largest block id of each table + 1: the smallest cache it may be used with
+    // u8 decode kernel: its split-K plan without / with scores (fixed per step) and, behind every table, the
+    // per-(sequence, split) descriptors of both plans
+    struct DecPlan { int32_t nsplit = 1, max_tiles = 1, waves = 4; } dec_plan[2];
+    size_t desc_off[2] = {0, 0};       // byte offsets of the two descriptor arrays in a table's buffer
+    std::vector<uint8_t> table_staging;
     bool shared_table = true;
     // workspace
     DevBuf part_acc, part_ml, final_ml, logits, group_scores, p_split, pf_part_acc, pf_part_ml;
@@ -192,16 +198,53 @@ const int32_t* table_for(pa_ctx* ctx, int32_t layer) {
     return ctx->tables[idx].as<int32_t>();
 }
 
-void check_io(pa_ctx* ctx, const pa_layer_io* io, bool need_kv, bool need_q) {
+void check_io(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool need_kv, bool need_q) {
     PA_REQUIRE(io, PA_INVALID_C_PARAM, "io is null");
     PA_REQUIRE(ctx->step_ready, PA_PARAMETER_MISMATCH, "pa_step_begin has not been called");
     PA_REQUIRE(io->key_cache && io->value_cache && io->num_blocks > 0, PA_INVALID_C_PARAM, "cache tensors missing");
+    // the table was validated against the num_blocks of its own call; the cache handed over now must hold its ids too
+    (void)table_for(ctx, layer);
+    PA_REQUIRE(io->num_blocks >= ctx->table_bound[ctx->shared_table ? 0 : (size_t)layer], PA_OUT_OF_BOUNDS,
+               "the cache tensors hold fewer blocks than the block table of this layer refers to");
     if (need_kv) PA_REQUIRE(io->key && io->value, PA_INVALID_C_PARAM, "key/value missing");
     if (need_q) PA_REQUIRE(io->query && io->out, PA_INVALID_C_PARAM, "query/out missing");
 }
 
+// Descriptors of the u8 decode kernel's workgroups for one block table (host ids), both plans, into the staging copy
+// of the table's buffer.
+void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
+    const int32_t sw = ctx->sliding_window;
+    std::vector<int32_t> soff(ctx->B + 1, 0);
+    for (int32_t b = 0; b < ctx->B; ++b) soff[b + 1] = soff[b] + ctx->h_past[b] + (ctx->h_sb[b + 1] - ctx->h_sb[b]);
+    for (int w = 0; w < 2; ++w) {
+        const int32_t nsplit = ctx->dec_plan[w].nsplit;
+        pa::DecodeDesc* out = reinterpret_cast<pa::DecodeDesc*>(stage + ctx->desc_off[w]);
+        for (size_t i = 0; i < ctx->h_dec.size(); ++i) {
+            const int32_t b = ctx->h_dec[i];
+            const int32_t kv_len = ctx->h_past[b] + 1;
+            const int32_t first = sw > 0 ? std::max(0, kv_len - sw) : 0;
+            const int32_t lo = first / 32, hi = (kv_len + 31) / 32;
+            const int32_t per = (hi - lo + nsplit - 1) / nsplit;
+            const int32_t* tab = ids + ctx->h_bib[b];
+            for (int32_t s = 0; s < nsplit; ++s) {
+                pa::DecodeDesc& d = out[i * nsplit + s];
+                d.b = b;
+                d.t = ctx->h_sb[b];
+                d.kv_len = kv_len;
+                d.first = first;
+                d.tb = lo + s * per;
+                d.te = std::min(hi, d.tb + per);
+                d.table_off = ctx->h_bib[b];
+                d.score_off = soff[b];
+                d.last_id = tab[hi - 1];
+                for (int32_t j = 0; j < 16; ++j) d.ids[j] = d.tb + j < d.te ? tab[d.tb + j] : 0;
+            }
+        }
+    }
+}
+
 void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
-    check_io(ctx, io, true, false);
+    check_io(ctx, layer, io, true, false);
     const int32_t* table = table_for(ctx, layer);
     HIP_CHECK(pa::launch_kv_append(ctx->stream, ctx->dev, shape_of(ctx->cfg), ctx->cfg.query_dtype,
                                    ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
@@ -420,6 +463,9 @@ void plan_items(pa_ctx* ctx) {
     }
     HIP_CHECK(hipStreamSynchronize(ctx->stream));
     ctx->tok_nsplit_off = item_bytes;
+    if (split_off_decode && !ctx->h_dec.empty())
+        for (int w = 0; w < 2; ++w)
+            plan_decode_u8(ctx, w == 1, &ctx->dec_plan[w].nsplit, &ctx->dec_plan[w].max_tiles, nullptr, &ctx->dec_plan[w].waves);
 }
 
 // Workspace of a decode launch (split partials, final maxima and denominators, per-kv-head score sums or per-head
@@ -473,8 +519,10 @@ DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_sc
     return w;
 }
 
-void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static_ws = false) {
-    check_io(ctx, io, false, true);
+// fuse_append: the call is the attention half of pa_forward in a step whose sequences all go to the u8 decode kernel,
+// and no append kernel has run: the decode kernel writes the step's K / V rows itself.
+void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static_ws = false, bool fuse_append = false) {
+    check_io(ctx, layer, io, false, true);
     const int32_t* table = table_for(ctx, layer);
     const pa_config& c = ctx->cfg;
     const size_t rows = (size_t)ctx->T * c.num_heads;
@@ -500,7 +548,14 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.G = c.num_heads / c.num_kv_heads;
         a.want_scores = io->scores ? 1 : 0;
         a.total_scores = ctx->total_scores;
-        plan_decode_u8(ctx, io->scores != nullptr, &a.nsplit, &a.max_tiles, nullptr, &a.waves);
+        const int wplan = io->scores ? 1 : 0;
+        a.nsplit = ctx->dec_plan[wplan].nsplit;
+        a.max_tiles = ctx->dec_plan[wplan].max_tiles;
+        a.waves = ctx->dec_plan[wplan].waves;
+        a.descs = reinterpret_cast<const pa::DecodeDesc*>(reinterpret_cast<const uint8_t*>(table) + ctx->desc_off[wplan]);
+        a.key = static_cast<const uint16_t*>(io->key);
+        a.value = static_cast<const uint16_t*>(io->value);
+        a.fuse_append = fuse_append ? 1 : 0;
         a.n_seqs = (int32_t)ctx->h_dec.size();
         a.seq_list = a.n_seqs == ctx->B ? nullptr : ctx->dec_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
@@ -791,8 +846,11 @@ int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int
         PA_REQUIRE(layer >= -1 && layer < ctx->cfg.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
         PA_REQUIRE(count == ctx->total_block_ids, PA_PARAMETER_MISMATCH,
                    "block_indices length differs from block_indices_begins[B]");
-        for (int32_t i = 0; i < count; ++i)
+        int64_t bound = 0;
+        for (int32_t i = 0; i < count; ++i) {
             PA_REQUIRE(ids[i] >= 0 && ids[i] < num_blocks, PA_OUT_OF_BOUNDS, "block index outside the cache");
+            bound = std::max<int64_t>(bound, (int64_t)ids[i] + 1);
+        }
         const bool shared = layer < 0;
         if (ctx->tables.empty() || shared != ctx->shared_table) {
             ctx->shared_table = shared;
@@ -802,16 +860,31 @@ int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int
                 for (auto& t : ctx->tables) t.release();
                 ctx->tables.assign(n, DevBuf());
                 ctx->table_count.assign(n, -1);
+                ctx->table_bound.assign(n, 0);
             }
         }
         const size_t idx = shared ? 0 : (size_t)layer;
+        // one upload: the ids, then (u8 decode kernel) the descriptors of its single-token sequences for the plan
+        // without and the plan with scores
+        const size_t id_bytes = ((size_t)count * sizeof(int32_t) + 127) & ~(size_t)127;
+        size_t total = std::max<size_t>(id_bytes, 128);
+        const bool with_descs = decode_u8_shape(ctx->cfg) && !ctx->h_dec.empty();
+        if (with_descs)
+            for (int w = 0; w < 2; ++w) {
+                ctx->desc_off[w] = total;
+                total += ctx->h_dec.size() * ctx->dec_plan[w].nsplit * sizeof(pa::DecodeDesc);
+            }
+        std::vector<uint8_t>& stage = ctx->table_staging;
+        stage.assign(total, 0);
+        std::memcpy(stage.data(), ids, (size_t)count * sizeof(int32_t));
+        if (with_descs) fill_decode_descs(ctx, ids, stage.data());
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
-        ctx->tables[idx].reserve(std::max<size_t>(1, (size_t)count) * sizeof(int32_t));
-        HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, ids, (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice,
-                                 ctx->stream));
+        ctx->tables[idx].reserve(total);
+        HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, stage.data(), total, hipMemcpyHostToDevice, ctx->stream));
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->table_count[idx] = count;
+        ctx->table_bound[idx] = bound;
     });
 }
 
@@ -995,8 +1068,11 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
     if (!ctx) return PA_INVALID_C_PARAM;
     return guarded(ctx, [&] {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
-        do_kv_append(ctx, layer, io);
-        do_attention(ctx, layer, io);
+        // a step of single-token sequences over a u8 cache: the decode kernel appends the new rows itself
+        const bool fuse = ctx->step_ready && decode_u8_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B;
+        if (fuse) check_io(ctx, layer, io, true, false);
+        else do_kv_append(ctx, layer, io);
+        do_attention(ctx, layer, io, false, fuse);
     });
 }
 
@@ -1191,8 +1267,10 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         if (seqs.empty()) return;
         PA_REQUIRE(key_cache && diversity, PA_INVALID_C_PARAM, "null argument");
         PA_REQUIRE(out_total <= capacity, PA_OUT_OF_BOUNDS, "diversity output holds fewer values than the areas need");
-        // the areas' blocks must exist in the cache (the table was checked against num_blocks of its own call)
-        PA_REQUIRE(num_blocks > 0, PA_PARAMETER_MISMATCH, "empty cache");
+        // the areas' blocks must exist in the cache handed over now (the table was checked against the num_blocks of
+        // its own call)
+        PA_REQUIRE(num_blocks >= ctx->table_bound[tidx] && num_blocks > 0, PA_OUT_OF_BOUNDS,
+                   "the key cache holds fewer blocks than the block table of this layer refers to");
         HIP_CHECK(hipSetDevice(c.device));
         HIP_CHECK(hipStreamSynchronize(ctx->stream));  // the previous call's kernels may still read the sequence list
         const int chunks = pa::rkv_diversity_chunks(ev_max);

@@ -1,29 +1,9 @@
-"""Parity soak: many more random steps than the suite holds, through the C-ABI against the CPU checker.
-
-    python tests/soak_random_steps.py [--kind small|big|peaked|sparse|wide] [--cases N] [--seed S]
-
-Not collected by pytest (it runs for minutes); every mismatch is printed with the step's shape so that it can be
-added to ``SOAK_FINDS`` in ``test_gpu_paged_attention.py``.  ``small`` draws from the same generator as the suite's
-random steps, ``big`` from longer contexts and chunks (several KV ranges per row, more sequences), ``peaked`` scales
-the logits so that few tokens carry a row.  Odd cases get planted +-8 outliers (every ``peaked`` case does).
-``sparse`` draws block-sparse prefill steps (XAttention: random block size, stride, thresholds, chunks mixed with
-dense and single-token sequences) and runs the three-link check of ``test_gpu_xattention.py`` on each.
-``wide`` draws decode steps over u8 caches with at least 256 (sequence, kv head) pairs in which a few contexts are
-too long for a four-wave workgroup's LDS (the eight-wave plan of the u8 decode kernel).
-"""
-import argparse
-import os
-import sys
-import time
-
+"""Generators of random steps beyond the suite's own: longer contexts and chunks (``big``), logits scaled so that few
+tokens carry a row (``peaked``), decode steps that take the eight-wave plan of the u8 decode kernel (``wide``) and
+block-sparse prefill steps (``sparse``).  Used by ``test_gpu_soak_slice.py``."""
 import numpy as np
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.dirname(HERE))
-sys.path.insert(0, HERE)
-
-import harness as H  # noqa: E402
-import test_gpu_paged_attention as T  # noqa: E402
+import harness as H
 
 
 def big_case(rng, idx):
@@ -103,44 +83,3 @@ def sparse_case(rng, idx):
                             sliding_window=sw, score_aggregation_window=saw, scale=mult / np.sqrt(D))
     case["thresholds"], case["xb"], case["S"] = np.array(thr, np.float32), xb, S
     return case
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--kind", choices=["small", "big", "peaked", "sparse", "wide"], default="small")
-    ap.add_argument("--cases", type=int, default=300)
-    ap.add_argument("--seed", type=int, default=50000)
-    ap.add_argument("--no-scores", action="store_true", help="ask for no scores (other kernels take the single-token "
-                    "sequences of 16-bit caches then)")
-    args = ap.parse_args()
-    import torch
-    import __graft_entry__ as entry
-    pkg = entry.load_package()
-    assert torch.cuda.is_available(), "the soak needs the GPU"
-    dev = torch.device("cuda:0")
-    make = {"small": T._random_case, "big": big_case, "peaked": peaked_case, "sparse": sparse_case, "wide": wide_case}[args.kind]
-    if args.kind == "sparse":
-        import test_gpu_xattention as TX
-    bad, t0 = 0, time.time()
-    for i in range(args.cases):
-        seed = args.seed + i
-        if i % 50 == 0:
-            print("progress: case %d of %d, %d mismatches, %.0f s" % (i, args.cases, bad, time.time() - t0), flush=True)
-        case = make(np.random.default_rng(seed), seed)
-        try:
-            if args.kind == "sparse":
-                TX._check(pkg, dev, H.build_case(case, seed, outliers=bool(i % 2)), case["thresholds"], case["xb"], case["S"],
-                          min_decided=0.0)
-            else:
-                T._check(pkg, dev, case, seed, outliers=args.kind == "peaked" or bool(i % 2), want_scores=not args.no_scores)
-        except AssertionError as e:
-            bad += 1
-            print("MISMATCH", case["name"], "seed", seed, "past", case["past_lens"].tolist(), "new", case["new_lens"].tolist(),
-                  "sw", case["sliding_window"], "saw", case["score_aggregation_window"],
-                  "thr", case.get("thresholds"), str(e)[:200], flush=True)
-    print("soak done: %d cases, %d mismatches, %.1f s" % (args.cases, bad, time.time() - t0), flush=True)
-    sys.exit(1 if bad else 0)
-
-
-if __name__ == "__main__":
-    main()

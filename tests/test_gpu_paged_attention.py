@@ -286,6 +286,16 @@ def test_errors_are_reported_not_thrown_across_the_abi(pkg, dev):
         op.attention(q, kc, kc, q)
     with pytest.raises(pkg.PaError):
         pkg.PagedAttention(8, 3, 128)  # heads not a multiple of kv heads
+    # a table validated against a large cache, then a layer call with a smaller one: refused before any launch
+    op.set_block_indices([0, 1, 2, 40], num_blocks=64)
+    for call in (lambda: op.attention(q, kc, kc, q), lambda: op.kv_append(q[:, :256], q[:, :256], kc, kc),
+                 lambda: op.forward(q, q[:, :256], q[:, :256], kc, kc, q)):
+        with pytest.raises(pkg.PaError) as e:
+            call()
+        assert e.value.status == -6, str(e.value)
+    big = torch.zeros(41, 2, 32, 136, dtype=torch.uint8, device=dev)
+    op.attention(q, big, big, torch.zeros_like(q))  # 41 blocks hold id 40
+    op.synchronize()
 
 
 def test_full_size_cfg2_properties(pkg, dev):

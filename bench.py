@@ -24,12 +24,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 NUM_LAYERS_FOR_TOKS = 32  # Llama-3-8B depth: tok/s = batch / (32 * t_layer), attention only
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the readings of
-# a plain 1 GiB copy (the summaries under profiles/ name the commands).
-MEASURED_TRAFFIC_BYTES = {"llama3_8b_decode_u8_b64_ctx4096": 584.8e6,
-                          "llama3_8b_eviction_u8_b256_ctx8192": 4655.0e6,
-                          "long_context_decode_u8_b8_ctx32768": 594.3e6,
-                          "qwen25_7b_mixed_bf16": 723.2e6}
+# HBM bytes per launch of the dominant kernel: not measured by this script but read off rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of it, scaled by the readings of a plain 1 GiB copy; the summary file holds commands and readings.
+MEASURED_TRAFFIC = {
+    "llama3_8b_decode_u8_b64_ctx4096": (584.8e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
+    "llama3_8b_eviction_u8_b256_ctx8192": (4655.0e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
+    "long_context_decode_u8_b8_ctx32768": (594.3e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
+    "qwen25_7b_mixed_bf16": (723.2e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
+}
 
 
 def parse():
@@ -45,6 +47,12 @@ def parse():
     ap.add_argument("--no-scores", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline")
+    ap.add_argument("--settle-steps", type=int, default=2000,
+                    help="untimed steps run before the warmup so that the GPU's clocks have settled when the timed "
+                         "steps start (a few thousand steps are a few tenths of a second); reported in `config`")
+    ap.add_argument("--layers", type=int, default=32,
+                    help="decoder layers of the eviction leg of --config 4 (score registration and eviction run over "
+                         "every layer of every sequence in one call)")
     ap.add_argument("--diversity", type=int, default=0, metavar="TOKENS",
                     help="adds a leg: ADAPTIVE_RKV block diversity over an evictable area of this many tokens (a "
                          "multiple of 32) of every sequence, behind a start area of 32 tokens")
@@ -90,27 +98,15 @@ def fill_cache(torch, op, spec, kc, vc, dev, gen):
         op.synchronize()
 
 
-def cpu_baseline(spec, seconds, with_scores):
-    """Times the CPU checker on the same shapes (contents: random codes, plausible headers)."""
+def cpu_baseline(spec, seconds, with_scores, q, kc, vc):
+    """Times the CPU checker on the inputs of the GPU leg: the same query rows, caches (as the library's append
+    kernel quantised them) and block table, copied to the host."""
     from oracle import oracle as O
     threads = min(os.cpu_count() or 1, 16)
-    B, Hq, Hkv, D, bs = spec["B"], spec["Hq"], spec["Hkv"], spec["D"], spec["bs"]
-    rng = np.random.default_rng(0)
+    Hq, Hkv, D, bs = spec["Hq"], spec["Hkv"], spec["D"], spec["bs"]
     dt = {"f16": O.DT_F16, "bf16": O.DT_BF16, "u8": O.DT_U8}
-    rb = O.row_bytes(D, dt[spec["kv_dtype"]])
-    nb = int(spec["block_indices_begins"][-1])
-    table = rng.permutation(nb).astype(np.int32)  # a 1x pool is enough for the host run
-    shape = (nb, Hkv, bs, rb)
-    if spec["kv_dtype"] == "u8":
-        kc = rng.integers(0, 256, size=shape, dtype=np.uint8)
-        hdr = np.array([0.0627, 127.5], np.float32).view(np.uint8)
-        kc[..., :8] = hdr
-        vc = kc[::-1].copy()
-    else:
-        kc = O.to_bits(rng.standard_normal((nb * Hkv * bs, D)).astype(np.float32), dt[spec["kv_dtype"]]).view(np.uint8).reshape(shape)
-        vc = kc[::-1].copy()
-    T = int(spec["subsequence_begins"][-1])
-    q = O.to_bits(rng.standard_normal((T, Hq * D)).astype(np.float32), dt[spec["q_dtype"]])
+    table = spec["block_indices"]
+
     def timed(n_threads, budget):
         times = []
         t_start = time.perf_counter()
@@ -128,58 +124,90 @@ def cpu_baseline(spec, seconds, with_scores):
 
 
 def cpu_model():
+    """What /proc/cpuinfo says of the first CPU: model name, vendor, family / model / stepping, clock."""
+    want = ("model name", "vendor_id", "cpu family", "model", "stepping", "cpu MHz")
+    got = {}
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
-                if line.startswith("model name"):
-                    return line.split(":", 1)[1].strip()
+                if ":" not in line:
+                    if got:
+                        break
+                    continue
+                key, val = (x.strip() for x in line.split(":", 1))
+                if key in want and key not in got:
+                    got[key] = val
     except OSError:
-        pass
-    return "unknown"
+        return "unknown"
+    return "%s (%s, family %s model %s stepping %s, %s MHz)" % (
+        got.get("model name", "unknown"), got.get("vendor_id", "?"), got.get("cpu family", "?"), got.get("model", "?"),
+        got.get("stepping", "?"), got.get("cpu MHz", "?"))
 
 
-def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev):
-    """Score accumulation + eviction on the device for the scoring workload (one layer): the first registration
-    sees the whole 8193-token context of every sequence and evicts down to max_cache_size, later ones one token."""
+def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, layers):
+    """Score accumulation + eviction on the device for the scoring workload, every layer of every sequence in one
+    call (the layers share one scores tensor here): the first registration sees the whole 8193-token context and
+    evicts down to max_cache_size; the steady state registers a 1024-token cache's scores and evicts one block.
+    Times are host wall clock around the C-ABI calls (upload of the per-pair entries, launches, read-back of the
+    evicted block lists included), buffers preallocated."""
+    import ctypes as C
+    from openvino_genai_amd import _lib as L
     B, bs = spec["B"], spec["bs"]
     cfg = pkg.CacheEvictionConfig(32, 128, 1024, pkg.AggregationMode.NORM_SUM, False, 0)
-    ev = pkg.Evictor(cfg, bs, 1, 7, max_sequences=B, max_tracked_tokens=8448, device=0,
+    ev = pkg.Evictor(cfg, bs, layers, 7, max_sequences=B, max_tracked_tokens=8448, device=0,
                      stream=torch.cuda.current_stream(dev))
-    slots = np.arange(B)
+    lib = L.lib()
+    slots = np.arange(B, dtype=np.int32)
+    ptrs = (C.c_void_p * layers)(*[C.c_void_p(scores.data_ptr())] * layers)
+    counts = np.zeros(B * layers, np.int32)
+    blocks = np.zeros(B * layers * 256, np.int32)
+    p32 = lambda a: a.ctypes.data_as(C.POINTER(C.c_int32))
+
+    def register(offsets):
+        L.check(lib.pa_evictor_register_scores(ev._h, B, p32(slots), ptrs, offsets.ctypes.data_as(C.POINTER(C.c_int64)), None),
+                lib.pa_evictor_last_error, ev._h)
+
+    def evict():
+        L.check(lib.pa_evictor_evict(ev._h, B, p32(slots), p32(counts), p32(blocks), 256), lib.pa_evictor_last_error, ev._h)
+
     kv = spec["past_lens"].astype(np.int64) + 1
-    offsets = np.concatenate([[0], np.cumsum(kv)])
+    offsets = np.concatenate([[0], np.cumsum(kv)]).astype(np.int64)
     op.attention(q, kc, vc, out, scores)
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
-    ev.register_new_token_scores(slots, [scores.data_ptr()], offsets, None)
+    register(offsets)
     torch.cuda.synchronize(dev)
     t1 = time.perf_counter()
-    got = ev.evict_logical_blocks(slots, max_blocks_per_entry=256)
+    evict()
     torch.cuda.synchronize(dev)
     t2 = time.perf_counter()
-    tracked = int((kv - 32).sum())
+    first_counts = counts.copy()
+    tracked = int((kv - 32).sum()) * layers
     # steady state: one more token per sequence on a 1024-token cache (scores of the capped context)
     kv2 = np.full(B, 1056 - 32 + 1 + 32, np.int64)
-    off2 = np.concatenate([[0], np.cumsum(kv2)])
-    reg, evi = [], []
-    for _ in range(8):
+    reg, evi, both = [], [], []
+    for _ in range(12):
+        off2 = np.concatenate([[0], np.cumsum(kv2)]).astype(np.int64)
         a = time.perf_counter()
-        ev.register_new_token_scores(slots, [scores.data_ptr()], off2, None)
-        torch.cuda.synchronize(dev)
-        b_ = time.perf_counter()
-        ev.evict_logical_blocks(slots, max_blocks_per_entry=256)
-        torch.cuda.synchronize(dev)
-        evi.append(time.perf_counter() - b_)
+        register(off2)
+        b_ = time.perf_counter()   # (the registration is left in flight: the eviction follows on the same stream)
+        evict()
+        c_ = time.perf_counter()
         reg.append(b_ - a)
+        evi.append(c_ - b_)
+        both.append(c_ - a)
         kv2 = kv2 + 1
-        off2 = np.concatenate([[0], np.cumsum(kv2)])
-    return {"first_register_ms": round((t1 - t0) * 1e3, 3), "first_evict_ms": round((t2 - t1) * 1e3, 3),
+    torch.cuda.synchronize(dev)
+    return {"layers": layers, "sequences": B,
+            "first_register_ms": round((t1 - t0) * 1e3, 3), "first_evict_ms": round((t2 - t1) * 1e3, 3),
             "first_register_GBps": round(tracked * 20 / (t1 - t0) / 1e9, 1),
-            "blocks_evicted_per_sequence_first": len(got[0][0]),
-            "steady_register_ms": round(float(np.median(reg)) * 1e3, 3),
-            "steady_evict_ms": round(float(np.median(evi)) * 1e3, 3),
-            "note": "host-side wall clock per call incl. upload of the per-sequence entries and the read-back of "
-                    "the evicted block lists; one layer, 256 sequences"}
+            "blocks_evicted_per_sequence_and_layer_first": [int(first_counts.min()), int(first_counts.max())],
+            "steady_register_call_ms": round(float(np.median(reg)) * 1e3, 3),
+            "steady_evict_call_ms": round(float(np.median(evi)) * 1e3, 3),
+            "steady_register_plus_evict_ms": round(float(np.median(both)) * 1e3, 3),
+            "note": "host wall clock per C-ABI call, %d sequences x %d layers per call; the steady-state pair is timed "
+                    "as one (register returns with its kernel in flight, evict returns with the block lists on the "
+                    "host); first_register_GBps prices 20 bytes per tracked token (4 read, 16 written)" % (B, layers)}
 
 
 def diversity_leg(torch, op, spec, kc, dev, ev, reps=20):
@@ -331,6 +359,9 @@ def main():
     def step():
         op.forward(q, k, v, kc, vc, out, scores)
 
+    for _ in range(args.settle_steps):  # clocks settle; not part of the warmup, not timed
+        step()
+    torch.cuda.synchronize(dev)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize(dev)
@@ -356,8 +387,9 @@ def main():
         cold_ms.append(op.last_kernel_ms())
     del flush
     op.set_profiling(False)
-    attn_ms = float(np.mean(kernel_ms))
     p10, p50, p90 = (float(x) for x in np.percentile(kernel_ms, [10, 50, 90]))
+    attn_ms = p50  # the roofline figures price the median launch
+    attn_mean_ms = float(np.mean(kernel_ms))
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -370,6 +402,8 @@ def main():
     gbps = bytes_["total"] / (ms_per_step * 1e-3) / 1e9
     attn_gbps = bytes_["total"] / (attn_ms * 1e-3) / 1e9
     mixed = T > B  # multi-token sequences present: the MFMA kernel is the dominant one
+    traffic, traffic_source = MEASURED_TRAFFIC.get(spec["name"], (None, None)) \
+        if with_scores and args.batch is None and not args.kv_dtype else (None, None)
     flops = wl.attention_flops(spec)
     res = {
         "metric": "paged-attn decode GB/s (tok/s and % HBM peak alongside), Llama-3-8B shape, u8 KV, 1 GPU"
@@ -380,24 +414,26 @@ def main():
         "dtype": spec["kv_dtype"] + "/f32", "data": "synthetic",
         "config": {"workload": spec["name"], "batch": B, "context": int(spec["past_lens"].max()) + 1,
                    "heads": [Hq, Hkv, D], "block_size": bs, "scores": with_scores, "splits": op.num_splits,
-                   "sliding_window": spec["sliding_window"]},
+                   "sliding_window": spec["sliding_window"], "clock_settle_steps": args.settle_steps},
         "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tok_per_s": round(B / (NUM_LAYERS_FOR_TOKS * ms_per_step * 1e-3), 1),
         "algorithmic_bytes": bytes_,
         "roofline": {"bound": "mfma", "kernel": "pa_prefill16_kernel", "achieved": round(flops / (attn_ms * 1e-3) / 1e12, 2),
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": round(flops / (attn_ms * 1e-3) / 1e12 / 2500.0, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(spec["name"]) if with_scores and args.batch is None and not args.kv_dtype else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "ms": round(attn_ms, 5), "flops": flops,
                      "hbm_GBps": round(bytes_["total"] / (attn_ms * 1e-3) / 1e9, 1)} if mixed else
                     {"bound": "hbm", "kernel": "pa_decode_u8_kernel" if spec["kv_dtype"] == "u8" else
                      ("pa_prefill16_kernel" if Hq // Hkv > 16 else "pa_decode16_kernel"), "achieved": round(attn_gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(attn_gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(spec["name"]) if with_scores and args.batch is None and not args.kv_dtype else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "ms": round(attn_ms, 5)},
     }
     res["roofline"]["ms_p10_p50_p90"] = [round(p10, 5), round(p50, 5), round(p90, 5)]
+    res["roofline"]["ms_mean"] = round(attn_mean_ms, 5)
+    res["roofline"]["launches"] = len(kernel_ms)
     if cold_ms:
-        cold = float(np.mean(cold_ms))
+        cold = float(np.median(cold_ms))
         res["roofline"]["cold"] = {"ms": round(cold, 5), "flush_mb": args.flush_mb,
                                    "frac": round(flops / (cold * 1e-3) / 1e12 / 2500.0, 4) if mixed else
                                    round(bytes_["total"] / (cold * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
@@ -406,11 +442,14 @@ def main():
     if args.diversity > 0:
         res["adaptive_rkv_diversity"] = diversity_leg(torch, op, spec, kc, dev, args.diversity)
     if args.config == 4:
-        res["eviction"] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev)
+        res["eviction"] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers)
     if not args.no_cpu_baseline:
-        t_cpu, n_pass, threads, t_one = cpu_baseline(spec, args.cpu_seconds, with_scores)
+        from oracle import oracle as O
+        q_h = q.view(torch.int16).cpu().numpy().view(np.uint16)
+        t_cpu, n_pass, threads, t_one = cpu_baseline(spec, args.cpu_seconds, with_scores, q_h, kc.cpu().numpy(), vc.cpu().numpy())
         res["cpu_baseline"] = {"value": round(bytes_["total"] / t_cpu / 1e9, 3), "unit": "GB/s", "cores": threads,
-                               "kind": "port", "sample": "the full batch of this workload, mean of %d passes of the "
+                               "kind": "port", "sample": "the full batch of this workload on the GPU leg's own inputs "
+                               "(query, quantised caches and block table copied to the host), mean of %d passes of the "
                                "CPU checker over %.1f s (%.4f s per pass)" % (n_pass, n_pass * t_cpu, t_cpu),
                                "value_1_thread": round(bytes_["total"] / t_one / 1e9, 3), "cpu": cpu_model(),
                                "host_cpus": os.cpu_count()}

@@ -126,6 +126,11 @@ hipError_t launch_kv_append(hipStream_t s, const StepDev& st, const Shape& sh, i
                             const void* key, const void* value, void* key_cache, void* value_cache,
                             const int32_t* block_indices);
 
+// Copy-on-write: block pairs[2 i] -> pairs[2 i + 1] in each of the n_tensors tensors whose base addresses `bases`
+// lists (device arrays); one launch for all of them.
+hipError_t launch_copy_blocks(hipStream_t s, void* const* bases, int n_tensors, const int32_t* pairs, int count,
+                              size_t block_bytes);
+
 struct AttnWorkspace {
     float* part_acc;   // [T*Hq*nsplit, D]
     float* part_ml;    // [T*Hq*nsplit, 2]

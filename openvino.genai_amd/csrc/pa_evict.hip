@@ -3,10 +3,14 @@
 // Per tracked sequence (slot) and decoder layer the library keeps `double scores[cap]` and
 // `uint64 counters[cap]`.  Three kernels:
 //   evict_register_kernel : forward max-pool of the op's f32 scores + accumulate (+ lifetime counters)
-//   evict_block_score / evict_rank / evict_list : per-block importance (sum of score / counter),
-//                           rank selection of the k lowest with ties to the lower index, ascending
-//                           list of evicted blocks
-//   evict_compact_kernel  : drops the evicted blocks' entries in place
+//   evict_select_compact_kernel : one workgroup per (sequence, layer), everything an eviction of the plain
+//                           modes needs in one launch: per-token score / counter staged through LDS (coalesced
+//                           reads), per-block importance summed in token order, rank selection of the k lowest
+//                           with ties to the lower index, the ascending list of evicted blocks, and the removal
+//                           of their entries in place
+//   evict_block_score / evict_rank / evict_list / evict_compact : the same steps as separate kernels, for the
+//                           modes whose choice among blocks runs on the host in between (ADAPTIVE_RKV, KVCrush)
+//                           and for areas too long for LDS
 //   evict_rkv_push / evict_rkv_mean_pool : ADAPTIVE_RKV tracker -- the last `window` score vectors are kept
 //                           in a ring per (slot, layer); the tracked score is their mean, max-pooled
 //   evict_filtered_diversity_kernel : per block row of a registered diversity matrix, the mean over the
@@ -64,7 +68,7 @@ struct SelEntry {       // one (sequence, layer) of an evict / remove call
     int32_t len;        // tracked tokens
     int32_t n_blocks;   // evictable blocks (from tracked block 0)
     int32_t k;          // blocks to evict
-    int32_t pad;
+    int32_t out_off;    // first entry of this pair's evicted blocks in the packed output (prefix sum of k)
 };
 
 __global__ __launch_bounds__(256) void evict_register_kernel(const RegEntry* __restrict__ entries,
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(256) void evict_block_score_kernel(const SelEntry* 
             const long t = e.state_off + (long)i * bsz + j;
             acc += norm_sum ? scores[t] / (double)counters[t] : scores[t];
         }
-        bscore[i] = acc;
+        bscore[i] = acc != acc ? INFINITY : acc;  // a block whose score is not a number is never preferred
     }
 }
 
@@ -199,6 +203,108 @@ __global__ __launch_bounds__(256) void evict_compact_kernel(const SelEntry* __re
         }
         __syncthreads();
     }
+}
+
+// Bytes of LDS the fused kernel needs for an entry: quotients [n_blocks][bsz + 1] doubles (the odd row length
+// keeps the per-block sums free of bank conflicts), block scores, flags, the evicted list.
+inline size_t select_lds_bytes(int64_t n_blocks, int64_t bsz, int64_t k) {
+    return (size_t)(n_blocks * (bsz + 1) * 8 + n_blocks * 8 + n_blocks * 4 + ((k + 1) & ~1LL) * 4);
+}
+
+// One workgroup per entry: block scores, selection, list and compaction.  `lds_blocks` is the largest n_blocks of
+// the launch (it fixes the carve-up); entries with k == 0 return at once.
+__global__ __launch_bounds__(256) void evict_select_compact_kernel(const SelEntry* __restrict__ entries,
+                                                                   double* __restrict__ scores,
+                                                                   unsigned long long* __restrict__ counters,
+                                                                   int32_t* __restrict__ out_list, int32_t bsz,
+                                                                   int32_t norm_sum, int32_t lds_blocks) {
+#pragma clang fp contract(off)
+    extern __shared__ __align__(16) uint8_t sel_smem[];
+    const SelEntry e = entries[blockIdx.x];
+    if (e.k <= 0 || e.n_blocks <= 0) return;
+    double* q = reinterpret_cast<double*>(sel_smem);                // [n_blocks][bsz + 1]
+    double* bscore = q + (size_t)lds_blocks * (bsz + 1);            // [n_blocks]
+    int32_t* flag = reinterpret_cast<int32_t*>(bscore + lds_blocks);  // [n_blocks]
+    int32_t* list = flag + lds_blocks;                              // [k]
+    const int tid = threadIdx.x;
+    const int n_tok = e.n_blocks * bsz;
+    for (int i = tid; i < n_tok; i += 256) {
+        const long t = e.state_off + i;
+        q[(i / bsz) * (bsz + 1) + i % bsz] = norm_sum ? scores[t] / (double)counters[t] : scores[t];
+    }
+    __syncthreads();
+    for (int i = tid; i < e.n_blocks; i += 256) {
+        double acc = 0.0;
+        for (int j = 0; j < bsz; ++j) acc += q[i * (bsz + 1) + j];
+        bscore[i] = acc != acc ? INFINITY : acc;  // a block whose score is not a number is never preferred
+    }
+    __syncthreads();
+    for (int i = tid; i < e.n_blocks; i += 256) {
+        const double si = bscore[i];
+        int rank = 0;
+        for (int j = 0; j < e.n_blocks; ++j) {
+            const double sj = bscore[j];
+            rank += (sj < si || (sj == si && j < i)) ? 1 : 0;
+        }
+        flag[i] = rank < e.k ? 1 : 0;
+    }
+    __syncthreads();
+    for (int i = tid; i < e.n_blocks; i += 256) {
+        if (!flag[i]) continue;
+        int pos = 0;
+        for (int j = 0; j < i; ++j) pos += flag[j];
+        list[pos] = i;
+        out_list[e.out_off + pos] = i;
+    }
+    __syncthreads();
+    // removal in place: chunks are read whole before any of their elements is written, and an element only ever
+    // moves towards lower indices
+    constexpr int PER = 4;
+    for (int base = 0; base < e.len; base += 256 * PER) {
+        double sv[PER];
+        unsigned long long cv[PER];
+        int dst[PER];
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int t = base + r * 256 + tid;
+            dst[r] = -1;
+            if (t < e.len) {
+                const int blk = t / bsz;
+                int lo = 0, hi = e.k;  // first list entry >= blk
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (list[mid] < blk) lo = mid + 1; else hi = mid;
+                }
+                const bool gone = lo < e.k && list[lo] == blk;
+                if (!gone) {
+                    dst[r] = t - lo * bsz;
+                    sv[r] = scores[e.state_off + t];
+                    if (norm_sum) cv[r] = counters[e.state_off + t];
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            if (dst[r] >= 0 && dst[r] != base + r * 256 + tid) {
+                scores[e.state_off + dst[r]] = sv[r];
+                if (norm_sum) counters[e.state_off + dst[r]] = cv[r];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Token scores of the listed entries' evictable areas, packed one after the other (for the host's KVCrush step).
+struct GatherEntry {
+    int64_t state_off, dst_off;
+    int32_t n;
+    int32_t pad;
+};
+__global__ __launch_bounds__(256) void evict_gather_kernel(const GatherEntry* __restrict__ entries,
+                                                           const double* __restrict__ scores, double* __restrict__ out) {
+    const GatherEntry e = entries[blockIdx.y];
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < e.n; i += gridDim.x * 256) out[e.dst_off + i] = scores[e.state_off + i];
 }
 
 constexpr int RKV_MAX_WINDOW = 32;
@@ -302,6 +408,28 @@ __global__ __launch_bounds__(256) void evict_filtered_diversity_kernel(const Fil
     if (threadIdx.x == 0) out[e.list_off + row] = acc / (double)((int64_t)e.set_size * bsz);
 }
 
+// Pinned host memory that only ever grows (allocated, never registered).
+struct PinnedBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    void reserve(size_t bytes) {
+        if (bytes <= cap) return;
+        if (p) HIP_CHECK(hipHostFree(p));
+        p = nullptr;
+        cap = 0;
+        const size_t want = std::max<size_t>(bytes + bytes / 2, 4096);
+        HIP_CHECK(hipHostMalloc(&p, want, hipHostMallocDefault));
+        cap = want;
+    }
+    void release() {
+        if (p) (void)hipHostFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <class T>
+    T* as() const { return static_cast<T*>(p); }
+};
+
 struct DevBuf {
     void* p = nullptr;
     size_t cap = 0;
@@ -335,7 +463,13 @@ struct pa_evictor {
     unsigned long long* counters = nullptr;
     std::vector<uint64_t> len;          // [slot * L + layer]
     std::vector<uint64_t> snapkv_seen;  // [slot]
-    DevBuf d_entries, d_ptrs, d_bscore, d_flags, d_list, d_filt;
+    DevBuf d_entries, d_ptrs, d_bscore, d_flags, d_list, d_filt, d_gather, d_gather_entries;
+    // pinned host staging: one buffer for what a call uploads, one for what it reads back; `staged` marks the end
+    // of the last upload from h_up (the buffer may be refilled once it has passed)
+    PinnedBuf h_up, h_back;
+    hipEvent_t staged = nullptr;
+    bool staged_pending = false;
+    std::vector<uint8_t> slot_mark;     // [max_sequences] scratch of the duplicate-slot check
     // ADAPTIVE_RKV: ring of the last `window` score vectors per (slot, layer)
     double* hist = nullptr;
     std::vector<int32_t> ring_len;    // [(slot * L + layer) * window + position]
@@ -454,6 +588,15 @@ pa_evictor* make(const pa_evictor_config* cfg, bool areas, uint64_t ignore_block
         delete ev;
         throw StatusError(PA_NOT_ALLOCATED, "not enough device memory for the eviction state");
     }
+    if (hipEventCreateWithFlags(&ev->staged, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(ev->scores);
+        (void)hipFree(ev->counters);
+        if (ev->hist) (void)hipFree(ev->hist);
+        delete ev;
+        throw StatusError(PA_GENERAL_ERROR, "could not create the staging event");
+    }
+    ev->slot_mark.assign(cfg->max_sequences, 0);
     const size_t pairs = (size_t)cfg->max_sequences * cfg->num_decoder_layers;
     ev->len.assign(pairs, 0);
     ev->snapkv_seen.assign(cfg->max_sequences, 0);
@@ -474,6 +617,40 @@ void upload(pa_evictor* ev, DevBuf& buf, const void* src, size_t bytes) {
     buf.reserve(bytes);
     HIP_CHECK(hipMemcpyAsync(buf.p, src, bytes, hipMemcpyHostToDevice, ev->stream));
     HIP_CHECK(hipStreamSynchronize(ev->stream));
+}
+
+// Pinned staging of what a call uploads: stage_begin hands out the buffer once the previous call's copy out of it has
+// passed, stage_copy enqueues a copy of a piece of it, stage_end marks the end of the call's copies.  Nothing waits for
+// the copies themselves: the kernels that read them follow on the same stream.
+uint8_t* stage_begin(pa_evictor* ev, size_t bytes) {
+    if (ev->staged_pending) {
+        HIP_CHECK(hipEventSynchronize(ev->staged));
+        ev->staged_pending = false;
+    }
+    ev->h_up.reserve(bytes);
+    return ev->h_up.as<uint8_t>();
+}
+void stage_copy(pa_evictor* ev, DevBuf& dst, size_t stage_off, size_t bytes) {
+    dst.reserve(bytes);
+    HIP_CHECK(hipMemcpyAsync(dst.p, ev->h_up.as<uint8_t>() + stage_off, bytes, hipMemcpyHostToDevice, ev->stream));
+}
+void stage_end(pa_evictor* ev) {
+    HIP_CHECK(hipEventRecord(ev->staged, ev->stream));
+    ev->staged_pending = true;
+}
+
+// Every slot of a call is in range and listed once.
+void check_slots(pa_evictor* ev, int32_t B, const int32_t* slots) {
+    bool twice = false;
+    int32_t i = 0;
+    for (; i < B; ++i) {
+        if (slots[i] < 0 || (uint64_t)slots[i] >= ev->cfg.max_sequences) break;
+        twice = twice || ev->slot_mark[slots[i]];
+        ev->slot_mark[slots[i]] = 1;
+    }
+    for (int32_t j = 0; j < i; ++j) ev->slot_mark[slots[j]] = 0;
+    PA_REQUIRE(i == B, PA_OUT_OF_BOUNDS, "slot out of range");
+    PA_REQUIRE(!twice, PA_PARAMETER_MISMATCH, "slot listed twice");
 }
 
 // Runs compaction for prepared entries whose evicted lists are already in d_list.
@@ -598,6 +775,11 @@ void pa_evictor_destroy(pa_evictor* ev) {
     ev->d_bscore.release();
     ev->d_flags.release();
     ev->d_list.release();
+    ev->d_gather.release();
+    ev->d_gather_entries.release();
+    ev->h_up.release();
+    ev->h_back.release();
+    if (ev->staged) (void)hipEventDestroy(ev->staged);
     delete ev;
 }
 
@@ -630,9 +812,8 @@ int32_t pa_evictor_register_scores(pa_evictor* ev, int32_t B, const int32_t* slo
         for (uint64_t l = 0; l < L; ++l) PA_REQUIRE(scores_per_layer[l], PA_INVALID_C_PARAM, "null scores pointer");
         // validate everything before touching state
         std::vector<uint64_t> seen(B);
+        check_slots(ev, B, slots);
         for (int32_t i = 0; i < B; ++i) {
-            check_slot(ev, slots[i]);
-            for (int32_t j = 0; j < i; ++j) PA_REQUIRE(slots[j] != slots[i], PA_PARAMETER_MISMATCH, "slot listed twice");
             PA_REQUIRE(offsets[i + 1] >= offsets[i], PA_PARAMETER_MISMATCH, "offsets must be non-decreasing");
             const uint64_t ns = num_snapkv ? num_snapkv[i] : 0;
             uint64_t s = ev->snapkv_seen[slots[i]];
@@ -689,14 +870,20 @@ int32_t pa_evictor_register_scores(pa_evictor* ev, int32_t B, const int32_t* slo
         }
         HIP_CHECK(hipSetDevice(ev->cfg.device));
         if (longest > 0) {
-            upload(ev, ev->d_entries, entries.data(), entries.size() * sizeof(RegEntry));
-            upload(ev, ev->d_ptrs, scores_per_layer, L * sizeof(float*));
+            // one pinned staging buffer (layer pointers | entries), two copies, one launch; nothing waits: whatever
+            // reads the state later follows on the same stream
+            const size_t ptr_bytes = (L * sizeof(float*) + 15) & ~(size_t)15, ent_bytes = entries.size() * sizeof(RegEntry);
+            uint8_t* st = stage_begin(ev, ptr_bytes + ent_bytes);
+            std::memcpy(st, scores_per_layer, L * sizeof(float*));
+            std::memcpy(st + ptr_bytes, entries.data(), ent_bytes);
+            stage_copy(ev, ev->d_ptrs, 0, L * sizeof(float*));
+            stage_copy(ev, ev->d_entries, ptr_bytes, ent_bytes);
+            stage_end(ev);
             dim3 grid((unsigned)std::min(pa::ceil_div(longest, 256), 64), (unsigned)B, (unsigned)L);
             hipLaunchKernelGGL(evict_register_kernel, grid, dim3(256), 0, ev->stream, ev->d_entries.as<RegEntry>(),
                                ev->d_ptrs.as<const float*>(), ev->scores, ev->counters, (int32_t)L,
                                (int32_t)ev->cfg.max_pool_window_size, norm ? 1 : 0);
             HIP_CHECK(hipGetLastError());
-            HIP_CHECK(hipStreamSynchronize(ev->stream));
         }
         for (int32_t i = 0; i < B; ++i) {
             ev->snapkv_seen[slots[i]] = seen[i];
@@ -715,9 +902,8 @@ int32_t pa_evictor_register_block_diversity(pa_evictor* ev, int32_t B, const int
         PA_REQUIRE(B > 0 && slots && diversity_per_layer && offsets, PA_INVALID_C_PARAM, "null argument");
         const uint64_t L = ev->L();
         for (uint64_t l = 0; l < L; ++l) PA_REQUIRE(diversity_per_layer[l], PA_INVALID_C_PARAM, "null diversity pointer");
+        check_slots(ev, B, slots);
         for (int32_t i = 0; i < B; ++i) {
-            check_slot(ev, slots[i]);
-            for (int32_t j = 0; j < i; ++j) PA_REQUIRE(slots[j] != slots[i], PA_PARAMETER_MISMATCH, "slot listed twice");
             PA_REQUIRE(offsets[i + 1] >= offsets[i], PA_PARAMETER_MISMATCH, "offsets must be non-decreasing");
             PA_REQUIRE(ev->div_off[slots[i]].empty(), PA_PARAMETER_MISMATCH,
                        "CacheEvictionAlgorithm already has block_diversity, must evict before new diversity is registered");
@@ -753,11 +939,11 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
         const bool rkv = ev->rkv();
         const bool crush = !rkv && ev->cfg.kvcrush_budget > 0;
         std::vector<SelEntry> entries((size_t)B * L);
-        int64_t list_total = 0;
+        int64_t list_total = 0, k_total = 0;
+        int32_t most_blocks_any = 0, most_k = 0;
         bool any = false;
+        check_slots(ev, B, slots);
         for (int32_t i = 0; i < B; ++i) {
-            check_slot(ev, slots[i]);
-            for (int32_t j = 0; j < i; ++j) PA_REQUIRE(slots[j] != slots[i], PA_PARAMETER_MISMATCH, "slot listed twice");
             for (uint64_t l = 0; l < L; ++l) {
                 SelEntry& e = entries[(size_t)i * L + l];
                 e = SelEntry{ev->state_off(slots[i], l), list_total, (int32_t)ev->len[(uint64_t)slots[i] * L + l], 0, 0, 0};
@@ -777,19 +963,26 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
                         e.k = (int32_t)ev->num_to_evict(re - rb);
                         PA_REQUIRE(e.k <= max_per_entry, PA_OUT_OF_BOUNDS, "more evicted blocks than the output holds");
                         any = any || e.k > 0;
+                        e.out_off = (int32_t)k_total;
+                        k_total += e.k;
+                        PA_REQUIRE(k_total <= INT32_MAX, PA_OUT_OF_BOUNDS, "too many evicted blocks for one call");
+                        if (e.k > 0) most_blocks_any = std::max(most_blocks_any, e.n_blocks);
+                        most_k = std::max(most_k, e.k);
                     }
                     list_total += e.n_blocks;
                 }
             }
         }
-        auto finish = [&](const std::vector<int32_t>& lists) {
+        // lists: per pair at list_off (one entry per evictable block) or, packed, at out_off (one per evicted block)
+        auto finish = [&](const int32_t* lists, bool packed) {
             const int32_t shift = (int32_t)(ev->cfg.start_size / bsz);
             for (int32_t i = 0; i < B; ++i) {
                 for (uint64_t l = 0; l < L; ++l) {
                     const SelEntry& e = entries[(size_t)i * L + l];
                     counts[(size_t)i * L + l] = e.k;
+                    const int32_t* mine = lists + (packed ? (size_t)e.out_off : (size_t)e.list_off);
                     for (int32_t p = 0; p < e.k; ++p)
-                        blocks[((size_t)i * L + l) * max_per_entry + p] = lists[(size_t)e.list_off + p] + shift;
+                        blocks[((size_t)i * L + l) * max_per_entry + p] = mine[p] + shift;
                     ev->len[(uint64_t)slots[i] * L + l] -= (uint64_t)e.k * bsz;
                     if (rkv && e.k > 0) ev->clear_ring(slots[i], l);  // remove_scores drops the history, :50
                 }
@@ -797,11 +990,33 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             }
         };
         if (!any) {
-            finish({});
+            finish(nullptr, false);
             return;
         }
         HIP_CHECK(hipSetDevice(ev->cfg.device));
         const int32_t norm = ev->cfg.aggregation_mode == PA_AGG_NORM_SUM ? 1 : 0;
+        const size_t fused_lds = select_lds_bytes(most_blocks_any, (int64_t)bsz, most_k);
+        if (!rkv && !crush && fused_lds <= 150 * 1024) {
+            // the plain modes: one upload, one launch (scores, selection, list, removal), one read-back
+            const size_t ent_bytes = entries.size() * sizeof(SelEntry);
+            uint8_t* st = stage_begin(ev, ent_bytes);
+            std::memcpy(st, entries.data(), ent_bytes);
+            stage_copy(ev, ev->d_entries, 0, ent_bytes);
+            stage_end(ev);
+            ev->d_list.reserve((size_t)k_total * sizeof(int32_t));
+            ev->h_back.reserve((size_t)k_total * sizeof(int32_t));
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(evict_select_compact_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)fused_lds));
+            hipLaunchKernelGGL(evict_select_compact_kernel, dim3((unsigned)entries.size()), dim3(256), fused_lds, ev->stream,
+                               ev->d_entries.as<SelEntry>(), ev->scores, ev->counters, ev->d_list.as<int32_t>(),
+                               (int32_t)bsz, norm, most_blocks_any);
+            HIP_CHECK(hipGetLastError());
+            HIP_CHECK(hipMemcpyAsync(ev->h_back.p, ev->d_list.p, (size_t)k_total * sizeof(int32_t), hipMemcpyDeviceToHost,
+                                     ev->stream));
+            HIP_CHECK(hipStreamSynchronize(ev->stream));
+            finish(ev->h_back.as<int32_t>(), true);
+            return;
+        }
         upload(ev, ev->d_entries, entries.data(), entries.size() * sizeof(SelEntry));
         ev->d_bscore.reserve((size_t)list_total * sizeof(double));
         ev->d_flags.reserve((size_t)list_total * sizeof(int32_t));
@@ -876,16 +1091,39 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             HIP_CHECK(hipStreamSynchronize(ev->stream));
             lists_on_device = true;
             if (crush) {  // cache_eviction.cpp:367-398: some of the chosen blocks stay as representatives
-                std::vector<double> tok;
+                // the token scores of every pair that needs them come back in one packed read
+                std::vector<GatherEntry> gather;
+                std::vector<size_t> gather_of(entries.size(), SIZE_MAX);
+                int64_t packed = 0;
+                int32_t longest = 0;
+                for (size_t x = 0; x < entries.size(); ++x) {
+                    const SelEntry& e = entries[x];
+                    if (e.k <= 0 || (uint64_t)e.k < ev->cfg.kvcrush_budget) continue;
+                    gather_of[x] = gather.size();
+                    gather.push_back(GatherEntry{e.state_off, packed, (int32_t)((size_t)e.n_blocks * bsz), 0});
+                    packed += (int64_t)e.n_blocks * (int64_t)bsz;
+                    longest = std::max(longest, gather.back().n);
+                }
+                if (!gather.empty()) {
+                    upload(ev, ev->d_gather_entries, gather.data(), gather.size() * sizeof(GatherEntry));
+                    ev->d_gather.reserve((size_t)packed * sizeof(double));
+                    ev->h_back.reserve((size_t)packed * sizeof(double));
+                    hipLaunchKernelGGL(evict_gather_kernel, dim3((unsigned)std::min(pa::ceil_div(longest, 256), 32), (unsigned)gather.size()),
+                                       dim3(256), 0, ev->stream, ev->d_gather_entries.as<GatherEntry>(), ev->scores,
+                                       ev->d_gather.as<double>());
+                    HIP_CHECK(hipGetLastError());
+                    HIP_CHECK(hipMemcpyAsync(ev->h_back.p, ev->d_gather.p, (size_t)packed * sizeof(double), hipMemcpyDeviceToHost,
+                                             ev->stream));
+                    HIP_CHECK(hipStreamSynchronize(ev->stream));
+                }
                 for (size_t x = 0; x < entries.size(); ++x) {
                     SelEntry& e = entries[x];
-                    if (e.k <= 0 || (uint64_t)e.k < ev->cfg.kvcrush_budget) continue;
+                    if (gather_of[x] == SIZE_MAX) continue;
                     const size_t n_tok = (size_t)e.n_blocks * bsz;
-                    tok.resize(n_tok);
-                    HIP_CHECK(hipMemcpy(tok.data(), ev->scores + e.state_off, n_tok * sizeof(double), hipMemcpyDeviceToHost));
+                    const double* tok_data = ev->h_back.as<double>() + gather[gather_of[x]].dst_off;
                     int32_t* list = lists.data() + e.list_off;
                     const std::vector<size_t> chosen(list, list + e.k);
-                    const std::vector<size_t> stay = ev->crush[slots[x / L]].blocks_to_retain(n_tok, chosen, tok.data());
+                    const std::vector<size_t> stay = ev->crush[slots[x / L]].blocks_to_retain(n_tok, chosen, tok_data);
                     int32_t k = 0;
                     for (size_t b : chosen)
                         if (std::find(stay.begin(), stay.end(), b) == stay.end()) list[k++] = (int32_t)b;
@@ -900,7 +1138,7 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
         }
         compact(ev, entries);
         HIP_CHECK(hipStreamSynchronize(ev->stream));
-        finish(lists);
+        finish(lists.data(), false);
     });
 }
 

@@ -153,14 +153,26 @@ struct pa_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
 
+// Every tensor (K and V of every layer) is a reserved range of virtual addresses whose front is backed by physical
+// memory; growth maps more memory behind what is there, so a tensor's base address never changes and no block moves.
 struct pa_kv_cache {
     pa_config cfg{};
     std::string error;
     uint64_t num_blocks = 0;
-    std::vector<void*> key, value;
+    std::vector<void*> key, value;      // base addresses (fixed from creation on)
+    size_t granularity = 0;             // size of every physical piece: memory is mapped in equal, equally aligned pieces
+    size_t reserved = 0, mapped = 0;    // per tensor: bytes of address space / bytes backed by memory
+    struct Chunk {
+        hipMemGenericAllocationHandle_t handle;
+        size_t offset, bytes;
+    };
+    std::vector<std::vector<Chunk>> chunks;  // per tensor: 2 * layer + (0 = K, 1 = V)
+    DevBuf base_table;                  // the 2 * num_layers base addresses, for the copy kernel
+    DevBuf pairs;                       // (source, destination) list of one copy launch
     uint64_t layer_block_bytes() const {  // one block of K (or V) in one layer
         return (uint64_t)cfg.num_kv_heads * cfg.block_size * pa::row_bytes(cfg.head_size, cfg.kv_cache_dtype);
     }
+    void*& tensor(size_t t) { return (t & 1) ? value[t >> 1] : key[t >> 1]; }
 };
 
 namespace {
@@ -1334,26 +1346,89 @@ uint64_t pa_snapkv_num_scores(uint64_t window, uint64_t prompt_len, uint64_t sch
 }
 
 // ------------------------------------------------------------------------------------ KV cache tensors
+namespace {
+
+hipMemAllocationProp device_memory_prop(int device) {
+    hipMemAllocationProp prop{};
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = device;
+    return prop;
+}
+
+// Unmaps and releases the chunks of every tensor from index `from[t]` on.
+void drop_chunks(pa_kv_cache* c, const std::vector<size_t>& from) {
+    for (size_t t = 0; t < c->chunks.size(); ++t) {
+        auto& list = c->chunks[t];
+        while (list.size() > from[t]) {
+            const pa_kv_cache::Chunk& ch = list.back();
+            (void)hipMemUnmap(static_cast<uint8_t*>(c->tensor(t)) + ch.offset, ch.bytes);
+            (void)hipMemRelease(ch.handle);
+            list.pop_back();
+        }
+    }
+}
+
+void destroy_kv_cache(pa_kv_cache* c) {
+    (void)hipSetDevice(c->cfg.device);
+    (void)hipDeviceSynchronize();
+    drop_chunks(c, std::vector<size_t>(c->chunks.size(), 0));
+    for (size_t t = 0; t < 2 * c->key.size(); ++t)
+        if (c->tensor(t)) (void)hipMemAddressFree(c->tensor(t), c->reserved);
+    c->base_table.release();
+    c->pairs.release();
+    delete c;
+}
+
+}  // namespace
+
 int32_t pa_kv_cache_create(const pa_config* cfg, pa_kv_cache** out) {
     return guarded<NoObj>(nullptr, [&] {
         PA_REQUIRE(out, PA_INVALID_C_PARAM, "out is null");
         *out = nullptr;
         check_config(cfg);
+        HIP_CHECK(hipSetDevice(cfg->device));
         pa_kv_cache* c = new pa_kv_cache();
         c->cfg = *cfg;
+        const size_t n_tensors = 2 * (size_t)cfg->num_layers;
         c->key.assign(cfg->num_layers, nullptr);
         c->value.assign(cfg->num_layers, nullptr);
+        c->chunks.assign(n_tensors, {});
+        try {
+            PA_REQUIRE(c->layer_block_bytes() % 16 == 0, PA_NOT_IMPLEMENTED, "a block of one layer must be a multiple of 16 bytes");
+            const hipMemAllocationProp prop = device_memory_prop(cfg->device);
+            size_t reported = 0;
+            HIP_CHECK(hipMemGetAllocationGranularity(&reported, &prop, hipMemAllocationGranularityRecommended));
+            PA_REQUIRE(reported > 0, PA_GENERAL_ERROR, "the device reports no allocation granularity");
+            // address space for as much as the device could ever hold, shared evenly between the tensors
+            size_t free_b = 0, total_b = 0;
+            HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+            // A tensor's memory is mapped in pieces of one size, each at a multiple of that size: on this device pieces
+            // of differing sizes behind one another were refused now and then (hipMemSetAccess: invalid argument), and so
+            // were pieces at offsets aligned only to the 4 KiB the runtime reports; equal pieces never were.  The size is
+            // a power of two near 1/1024 of the tensor's address range, between 2 MiB and 64 MiB: at most about a
+            // thousand pieces per tensor (each costs about 60 us to create and map), at most one piece per tensor unused.
+            size_t piece = (size_t)2 << 20;
+            while (piece < ((size_t)64 << 20) && piece < total_b / n_tensors / 1024) piece *= 2;
+            PA_REQUIRE(piece % reported == 0, PA_GENERAL_ERROR, "unexpected allocation granularity");
+            c->granularity = piece;
+            c->reserved = (total_b / n_tensors + piece - 1) / piece * piece;
+            for (size_t t = 0; t < n_tensors; ++t)
+                HIP_CHECK(hipMemAddressReserve(&c->tensor(t), c->reserved, c->granularity, nullptr, 0));
+            std::vector<void*> bases(n_tensors);
+            for (size_t t = 0; t < n_tensors; ++t) bases[t] = c->tensor(t);
+            c->base_table.reserve(n_tensors * sizeof(void*));
+            HIP_CHECK(hipMemcpy(c->base_table.p, bases.data(), n_tensors * sizeof(void*), hipMemcpyHostToDevice));
+        } catch (...) {
+            destroy_kv_cache(c);
+            throw;
+        }
         *out = c;
     });
 }
 
 void pa_kv_cache_destroy(pa_kv_cache* c) {
-    if (!c) return;
-    (void)hipSetDevice(c->cfg.device);
-    (void)hipDeviceSynchronize();
-    for (void* p : c->key) if (p) (void)hipFree(p);
-    for (void* p : c->value) if (p) (void)hipFree(p);
-    delete c;
+    if (c) destroy_kv_cache(c);
 }
 
 const char* pa_kv_cache_last_error(const pa_kv_cache* c) { return c ? c->error.c_str() : g_last_error.c_str(); }
@@ -1370,24 +1445,53 @@ int32_t pa_kv_cache_allocate(pa_kv_cache* c, uint64_t num_kv_blocks) {
         if (c->num_blocks >= num_kv_blocks) return;
         HIP_CHECK(hipSetDevice(c->cfg.device));
         hipStream_t s = static_cast<hipStream_t>(c->cfg.stream);
+        const char* too_large = "Requested KV-cache size is larger than available memory size on the system.";
         const uint64_t bb = c->layer_block_bytes();
-        for (int32_t l = 0; l < c->cfg.num_layers; ++l) {
-            for (int which = 0; which < 2; ++which) {
-                void*& cur = which ? c->value[l] : c->key[l];
-                void* fresh = nullptr;
-                hipError_t e = hipMalloc(&fresh, num_kv_blocks * bb);
+        PA_REQUIRE(num_kv_blocks <= c->reserved / bb, PA_NOT_ALLOCATED, too_large);
+        const size_t need = ((size_t)(num_kv_blocks * bb) + c->granularity - 1) / c->granularity * c->granularity;
+        if (need > c->mapped) {
+            // memory for every tensor first, then the mappings: a failure anywhere leaves the cache as it was
+            const size_t add = need - c->mapped, n_tensors = c->chunks.size(), piece = c->granularity;
+            const size_t per_tensor = add / piece, n_fresh = per_tensor * n_tensors;
+            const hipMemAllocationProp prop = device_memory_prop(c->cfg.device);
+            std::vector<size_t> before(n_tensors);
+            for (size_t t = 0; t < n_tensors; ++t) before[t] = c->chunks[t].size();
+            std::vector<hipMemGenericAllocationHandle_t> fresh;
+            fresh.reserve(n_fresh);
+            for (size_t i = 0; i < n_fresh; ++i) {
+                hipMemGenericAllocationHandle_t h;
+                if (hipMemCreate(&h, piece, &prop, 0) != hipSuccess) {
+                    (void)hipGetLastError();
+                    for (auto& f : fresh) (void)hipMemRelease(f);
+                    throw StatusError(PA_NOT_ALLOCATED, too_large);
+                }
+                fresh.push_back(h);
+            }
+            hipMemAccessDesc access{};
+            access.location = prop.location;
+            access.flags = hipMemAccessFlagsProtReadWrite;
+            for (size_t i = 0; i < n_fresh; ++i) {
+                const size_t t = i / per_tensor, off = c->mapped + (i % per_tensor) * piece;
+                uint8_t* at = static_cast<uint8_t*>(c->tensor(t)) + off;
+                hipError_t e = hipMemMap(at, piece, 0, fresh[i], 0);
+                bool listed = false;
+                if (e == hipSuccess) {
+                    c->chunks[t].push_back({fresh[i], off, piece});
+                    listed = true;
+                    e = hipMemSetAccess(at, piece, &access, 1);
+                }
                 if (e != hipSuccess) {
                     (void)hipGetLastError();
-                    throw StatusError(PA_NOT_ALLOCATED,
-                                      "Requested KV-cache size is larger than available memory size on the system.");
+                    for (size_t u = listed ? i + 1 : i; u < n_fresh; ++u) (void)hipMemRelease(fresh[u]);
+                    drop_chunks(c, before);
+                    throw StatusError(PA_NOT_ALLOCATED, std::string("mapping KV-cache memory failed: ") + hipGetErrorString(e));
                 }
-                if (cur) {
-                    HIP_CHECK(hipMemcpyAsync(fresh, cur, c->num_blocks * bb, hipMemcpyDeviceToDevice, s));
-                    HIP_CHECK(hipStreamSynchronize(s));
-                    HIP_CHECK(hipFree(cur));
-                }
-                cur = fresh;
             }
+            // new blocks start as zeros (rows no token has been written to are then harmless in any format)
+            for (size_t t = 0; t < n_tensors; ++t)
+                HIP_CHECK(hipMemsetAsync(static_cast<uint8_t*>(c->tensor(t)) + c->mapped, 0, add, s));
+            HIP_CHECK(hipStreamSynchronize(s));
+            c->mapped = need;
         }
         c->num_blocks = num_kv_blocks;
     });
@@ -1408,19 +1512,42 @@ int32_t pa_kv_cache_copy_blocks(pa_kv_cache* c, const int32_t* src, const int32_
         for (int32_t i = 0; i < count; ++i)
             PA_REQUIRE(src[i] >= 0 && dst[i] >= 0 && (uint64_t)src[i] < c->num_blocks && (uint64_t)dst[i] < c->num_blocks,
                        PA_OUT_OF_BOUNDS, "block index outside the cache");
+        if (count == 0) return;
         HIP_CHECK(hipSetDevice(c->cfg.device));
         hipStream_t s = static_cast<hipStream_t>(c->cfg.stream);
-        const uint64_t bb = c->layer_block_bytes();
-        for (int32_t i = 0; i < count; ++i) {
-            if (src[i] == dst[i]) continue;
-            for (int32_t l = 0; l < c->cfg.num_layers; ++l) {
-                HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(c->key[l]) + dst[i] * bb,
-                                         static_cast<uint8_t*>(c->key[l]) + src[i] * bb, bb, hipMemcpyDeviceToDevice, s));
-                HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(c->value[l]) + dst[i] * bb,
-                                         static_cast<uint8_t*>(c->value[l]) + src[i] * bb, bb, hipMemcpyDeviceToDevice, s));
+        // The pairs of one launch are copied side by side, the reference copies them one after the other: a pair that
+        // reads what an earlier pair writes, or writes what an earlier pair reads or writes, starts a new launch.
+        std::vector<int32_t> list;
+        list.reserve(2 * (size_t)count);
+        std::vector<int32_t> cuts{0};  // first pair of every launch
+        {
+            std::vector<uint8_t> role(c->num_blocks, 0);  // 1 = read, 2 = written by the launch being formed
+            std::vector<int32_t> touched;
+            for (int32_t i = 0; i < count; ++i) {
+                if (src[i] == dst[i]) continue;
+                if (role[src[i]] == 2 || role[dst[i]] != 0) {
+                    for (int32_t b : touched) role[b] = 0;
+                    touched.clear();
+                    cuts.push_back((int32_t)(list.size() / 2));
+                }
+                role[src[i]] = std::max<uint8_t>(role[src[i]], 1);
+                role[dst[i]] = 2;
+                touched.push_back(src[i]);
+                touched.push_back(dst[i]);
+                list.push_back(src[i]);
+                list.push_back(dst[i]);
             }
         }
-        HIP_CHECK(hipStreamSynchronize(s));
+        if (list.empty()) return;
+        cuts.push_back((int32_t)(list.size() / 2));
+        HIP_CHECK(hipStreamSynchronize(s));  // an earlier call's launches may still read the list
+        c->pairs.reserve(list.size() * sizeof(int32_t));
+        HIP_CHECK(hipMemcpyAsync(c->pairs.p, list.data(), list.size() * sizeof(int32_t), hipMemcpyHostToDevice, s));
+        for (size_t k = 0; k + 1 < cuts.size(); ++k)
+            HIP_CHECK(pa::launch_copy_blocks(s, c->base_table.as<void*>(), (int)c->chunks.size(),
+                                             c->pairs.as<int32_t>() + 2 * cuts[k], cuts[k + 1] - cuts[k],
+                                             c->layer_block_bytes()));
+        HIP_CHECK(hipStreamSynchronize(s));  // `list` is pageable and leaves scope; the reference's copy is synchronous too
     });
 }
 

@@ -234,3 +234,103 @@ def test_decode_scores_feed_eviction_like_the_pipeline(pkg):
         past = past + 1 - n_ev * bs
     assert evicted_any
     assert all(p <= mx + bs for p in past)  # per-sequence cache stays capped (cache_eviction.cpp:297-303)
+
+
+@pytest.mark.parametrize("snapkv", [0, 8])
+def test_full_size_scoring_workload_eviction_matches_checker(pkg, snapkv):
+    """The scoring workload at full size: 256 sequences at 8192 tokens of context (Llama-3-8B shape, u8 KV, two
+    layers with their own caches and tables), real decode scores on the device -> register -> evict -> drop the
+    evicted blocks from the tables, for 34 consecutive steps (NORM_SUM, start 32 / recent 128 / max 1024, max-pool 7).
+    The checker's restatement of CacheEvictionAlgorithm is fed the same device scores: evicted lists, f64 scores and
+    u64 counters must be identical.  The first eviction frees 224 blocks per (sequence, layer); the second one
+    comes 31 steps later."""
+    import torch
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, D, bs, L = 256, 32, 8, 128, 32, 2
+    start, recent, mx = 32, 128, 1024
+    ctx0 = 8192
+    gen = torch.Generator(device=dev).manual_seed(1004 + snapkv)
+    rng = np.random.default_rng(1004 + snapkv)
+    nblk0 = ctx0 // bs + 1
+    pool = B * (nblk0 + 1)
+    caches = []
+    for l in range(L):
+        pair = []
+        for _ in range(2):
+            c = torch.randint(0, 256, (pool, Hkv, bs, D + 8), dtype=torch.uint8, device=dev, generator=gen)
+            hdr = torch.empty(pool, Hkv, bs, 2, dtype=torch.float32, device=dev)
+            hdr[..., 0] = 0.02 + 0.04 * torch.rand(pool, Hkv, bs, device=dev, generator=gen)
+            hdr[..., 1] = 100.0 + 50.0 * torch.rand(pool, Hkv, bs, device=dev, generator=gen)
+            c[..., :8] = hdr.view(torch.uint8).view(pool, Hkv, bs, 8)
+            pair.append(c)
+            del hdr
+        caches.append(pair)
+    perm = rng.permutation(pool)
+    tables = [[list(perm[b * (nblk0 + 1): b * (nblk0 + 1) + nblk0]) for b in range(B)] for _ in range(L)]
+    spare = [[int(perm[b * (nblk0 + 1) + nblk0])] for b in range(B)]   # one more block per sequence, for growth
+    cfg = pkg.CacheEvictionConfig(start, recent, mx, pkg.AggregationMode.NORM_SUM, False, snapkv)
+    ev = pkg.Evictor(cfg, bs, L, 7, max_sequences=B, max_tracked_tokens=ctx0 + 64, device=0,
+                     stream=torch.cuda.current_stream(dev))
+    refs = [O.CacheEvictionAlgorithm(start, recent, mx, O.MODE_NORM_SUM, snapkv, bs, L, 7) for _ in range(B)]
+    op = pkg.PagedAttention(Hq, Hkv, D, bs, "f16", "u8", num_layers=L, device=0, stream=torch.cuda.current_stream(dev))
+    past = np.full(B, ctx0, np.int64)
+    slots = np.arange(B, dtype=np.int32)
+    sb = np.arange(B + 1, dtype=np.int32)
+    evictions = []
+    for step in range(34):
+        for b in range(B):
+            if (past[b] + 1 + bs - 1) // bs > len(tables[0][b]):
+                blk = spare[b].pop()
+                for l in range(L):
+                    tables[l][b].append(blk)
+        q = torch.randn(B, Hq * D, device=dev, generator=gen).to(torch.float16)
+        k = torch.randn(B, Hkv * D, device=dev, generator=gen).to(torch.float16)
+        v = torch.randn(B, Hkv * D, device=dev, generator=gen).to(torch.float16)
+        bib = np.concatenate([[0], np.cumsum([len(t) for t in tables[0]])]).astype(np.int32)
+        op.step_begin(past.astype(np.int32), sb, bib)
+        scores = []
+        for l in range(L):
+            assert [len(t) for t in tables[l]] == [len(t) for t in tables[0]]
+            op.set_block_indices(np.concatenate(tables[l]).astype(np.int32), pool, layer=l)
+            out = torch.empty_like(q)
+            sc = torch.full((op.total_scores,), float("nan"), dtype=torch.float32, device=dev)
+            op.forward(q, k, v, caches[l][0], caches[l][1], out, sc, layer=l)
+            scores.append(sc)
+        op.synchronize()
+        offsets = np.concatenate([[0], np.cumsum(past + 1)]).astype(np.int64)
+        n_snap = np.full(B, 1 if snapkv else 0, np.uint64)   # generation phase: one score row per step
+        ev.register_new_token_scores(slots, [s.data_ptr() for s in scores], offsets, n_snap)
+        host = [s.cpu().numpy() for s in scores]
+        assert all(np.isfinite(h).all() for h in host)
+        for b in range(B):
+            refs[b].register_new_token_scores([h[offsets[b]:offsets[b + 1]] for h in host], (), int(n_snap[b]))
+        check_all = step in (0, 1, 7, 31, 32)
+        for b in (range(B) if check_all else (0, 97, 255)):
+            for l in range(L):
+                gs, gc = ev.get_state(b, l)
+                assert np.array_equal(gs, refs[b].get_scores()[l]), (step, b, l)
+                assert np.array_equal(gc, refs[b].get_counters()[l]), (step, b, l)
+        got = ev.evict_logical_blocks(slots, max_blocks_per_entry=256)
+        n_ev = np.zeros(B, np.int64)
+        for b in range(B):
+            exp = refs[b].evict_logical_blocks()
+            assert got[b] == exp, (step, b)
+            n_ev[b] = len(exp[0])
+            for l in range(L):
+                assert len(exp[l]) == n_ev[b]
+                for blk in sorted(exp[l], reverse=True):
+                    freed = tables[l][b].pop(blk)
+                    if l == 0:
+                        spare[b].append(int(freed))   # (layer 0's freed blocks serve as this sequence's growth pool)
+        if step in (0, 31):
+            for b in range(0, B, 17):
+                for l in range(L):
+                    gs, gc = ev.get_state(b, l)
+                    assert np.array_equal(gs, refs[b].get_scores()[l]) and np.array_equal(gc, refs[b].get_counters()[l])
+        evictions.append(n_ev.copy())
+        past = past + 1 - n_ev * bs
+    assert (evictions[0] == 224).all()            # 251 evictable blocks, 27 kept
+    # then one token per step: 1025 + k tokens at step k pass max_cache_size + block_size - 1 = 1055 at k = 31
+    assert all((e == 0).all() for e in evictions[1:31])
+    assert (evictions[31] == 1).all() and (evictions[32] == 0).all() and (evictions[33] == 0).all()
+    assert (past <= mx + bs).all()

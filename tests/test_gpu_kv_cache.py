@@ -134,3 +134,118 @@ def test_copy_blocks_and_use_as_op_tensors(env):
         assert np.array_equal(o1, o2) and np.array_equal(s1, s2)
     with pytest.raises(pkg.PaError):
         mgr.copy_blocks({0: [2 * nb]})  # outside the cache
+
+
+def test_growth_moves_nothing_and_new_blocks_are_zero(env):
+    """Growth maps memory behind what is there: base addresses stay, old blocks stay in place, new ones read as 0."""
+    pkg, _, hip = env
+    layers = 2
+    mgr = pkg.KVCacheManager(layers, 4, 128, 32, "u8")
+    per_layer = mgr.get_block_size_in_bytes() // (2 * layers)
+    mgr.allocate_cache_if_needed(7)
+    ptrs = [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(layers)]
+    rng = np.random.default_rng(5)
+    want = {}
+    for l in range(layers):
+        for w in range(2):
+            want[l, w] = rng.integers(0, 256, 7 * per_layer, dtype=np.uint8)
+            _write(hip, ptrs[l][w], want[l, w])
+    for n in (8, 300, 5000):   # within the first mapping's slack, then across several mappings
+        mgr.allocate_cache_if_needed(n)
+        assert [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(layers)] == ptrs
+        for l in range(layers):
+            for w in range(2):
+                got = _read(hip, ptrs[l][w], n * per_layer)
+                assert np.array_equal(got[:7 * per_layer], want[l, w]), (n, l, w)
+                assert not got[7 * per_layer:].any(), (n, l, w)
+
+
+def test_failed_growth_leaves_the_cache_as_it_was(env):
+    pkg, _, hip = env
+    mgr = pkg.KVCacheManager(2, 4, 128, 32, "u8")
+    per_layer = mgr.get_block_size_in_bytes() // 4
+    mgr.allocate_cache_if_needed(10)
+    ptr = mgr.get_key_cache(1)
+    data = np.arange(10 * per_layer, dtype=np.uint32).astype(np.uint8)
+    _write(hip, ptr, data)
+    with pytest.raises(pkg.PaError) as e:   # more than the device holds
+        mgr.allocate_cache_if_needed((400 << 30) // mgr.get_block_size_in_bytes())
+    assert e.value.status == -10 and "larger than available memory" in str(e.value)
+    assert mgr.get_num_allocated_kv_blocks() == 10 and mgr.get_key_cache(1) == ptr
+    assert np.array_equal(_read(hip, ptr, 10 * per_layer), data)
+    mgr.allocate_cache_if_needed(20)        # and it still grows
+    assert np.array_equal(_read(hip, ptr, 10 * per_layer), data)
+
+
+def test_growth_past_half_of_the_free_memory(env):
+    """From N to 2N blocks with N above a third of the free memory: a growth that copied into a new allocation could
+    not hold both; here nothing is copied, addresses stay valid and the contents stay where they are."""
+    import torch
+    pkg, dev, hip = env
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info(dev)
+    layers = 4
+    mgr = pkg.KVCacheManager(layers, 8, 128, 32, "u8")
+    bb = mgr.get_block_size_in_bytes()
+    per_layer = bb // (2 * layers)
+    n = int(0.36 * free) // bb
+    mgr.allocate_cache_if_needed(n)
+    ptrs = [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(layers)]
+    rng = np.random.default_rng(9)
+    marks = {}
+    for l in range(layers):
+        for w in range(2):
+            for blk in (0, n // 2, n - 1):
+                marks[l, w, blk] = rng.integers(0, 256, per_layer, dtype=np.uint8)
+                _write(hip, ptrs[l][w] + blk * per_layer, marks[l, w, blk])
+    mgr.allocate_cache_if_needed(2 * n)
+    assert mgr.get_num_allocated_kv_blocks() == 2 * n
+    assert 2 * n * bb > 0.7 * free
+    assert [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(layers)] == ptrs
+    for (l, w, blk), data in marks.items():
+        assert np.array_equal(_read(hip, ptrs[l][w] + blk * per_layer, per_layer), data), (l, w, blk)
+    last = ptrs[layers - 1][1] + (2 * n - 1) * per_layer
+    assert not _read(hip, last, per_layer).any()
+    _write(hip, last, marks[0, 0, 0])
+    assert np.array_equal(_read(hip, last, per_layer), marks[0, 0, 0])
+    del mgr
+    torch.cuda.synchronize(dev)
+    assert torch.cuda.mem_get_info(dev)[0] > 0.9 * free   # everything was given back
+
+
+def test_copy_blocks_of_a_whole_batch_is_exact_and_ordered(env):
+    """256 pairs x 32 layers in one call; then pairs that feed each other, which the reference copies one after the
+    other (kv_cache_manager.hpp:278-335)."""
+    import time
+    pkg, _, hip = env
+    layers = 32
+    mgr = pkg.KVCacheManager(layers, 8, 128, 32, "u8")
+    per_layer = mgr.get_block_size_in_bytes() // (2 * layers)
+    nb = 600
+    mgr.allocate_cache_if_needed(nb)
+    rng = np.random.default_rng(3)
+    content = {}
+    for l in range(layers):
+        for w in range(2):
+            content[l, w] = rng.integers(0, 256, (nb, per_layer), dtype=np.uint8)
+            _write(hip, (mgr.get_key_cache(l), mgr.get_value_cache(l))[w], content[l, w])
+    src = rng.permutation(300)[:256]
+    copy_map = {int(s): [300 + i] for i, s in enumerate(src)}
+    t0 = time.perf_counter()
+    mgr.copy_blocks(copy_map)
+    dt = time.perf_counter() - t0
+    print("copy_blocks: 256 blocks x 32 layers (%.0f MB read + written) in %.3f ms host time" %
+          (2 * 256 * mgr.get_block_size_in_bytes() / 1e6, dt * 1e3))
+    for l in (0, 13, 31):
+        for w in range(2):
+            got = _read(hip, (mgr.get_key_cache(l), mgr.get_value_cache(l))[w], nb * per_layer).reshape(nb, per_layer)
+            want = content[l, w].copy()
+            for s, ds in copy_map.items():
+                want[ds[0]] = content[l, w][s]
+            assert np.array_equal(got, want), (l, w)
+    # 0 -> 1, then 1 -> 2: block 2 ends up with what block 0 held; one source, several destinations
+    base0 = _read(hip, mgr.get_key_cache(5), 3 * per_layer).reshape(3, per_layer)
+    mgr.copy_blocks({0: [1, 590, 591], 1: [2]})
+    got = _read(hip, mgr.get_key_cache(5), nb * per_layer).reshape(nb, per_layer)
+    for blk in (1, 2, 590, 591):
+        assert np.array_equal(got[blk], base0[0]), blk

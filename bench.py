@@ -59,6 +59,8 @@ def parse():
     ap.add_argument("--xattention", type=float, default=0.0, metavar="THRESHOLD",
                     help="adds a leg: block-sparse prefill with this threshold against dense prefill (4 x 512-token "
                          "chunks, Qwen2.5-7B shape, bf16 cache)")
+    ap.add_argument("--kv-cache-leg", action="store_true",
+                    help="adds a leg: copy-on-write of 256 blocks x 32 layers and growth of the cache tensors")
     ap.add_argument("--pool-factor", type=float, default=2.0,
                     help="size of the block pool the tables are drawn from, as a multiple of the blocks in use")
     ap.add_argument("--flush-mb", type=int, default=1024,
@@ -208,6 +210,40 @@ def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, layers):
             "note": "host wall clock per C-ABI call, %d sequences x %d layers per call; the steady-state pair is timed "
                     "as one (register returns with its kernel in flight, evict returns with the block lists on the "
                     "host); first_register_GBps prices 20 bytes per tracked token (4 read, 16 written)" % (B, layers)}
+
+
+def kv_cache_leg(torch, pkg, dev, layers=32, blocks=256):
+    """Block-table maintenance on the device: copy-on-write of `blocks` blocks in every layer's K and V tensor (one
+    call), and growth of the cache from N to 2N blocks (Llama-3-8B shape, u8).  Host wall clock around the
+    synchronous C-ABI calls."""
+    mgr = pkg.KVCacheManager(layers, 8, 128, 32, "u8")
+    bb = mgr.get_block_size_in_bytes()
+    n = 4 * blocks
+    t0 = time.perf_counter()
+    mgr.allocate_cache_if_needed(n)
+    t1 = time.perf_counter()
+    first_ptr = mgr.get_key_cache(0)
+    times = []
+    for r in range(6):
+        copy_map = {int(i): [2 * blocks + (int(i) + r) % blocks] for i in range(blocks)}
+        a = time.perf_counter()
+        mgr.copy_blocks(copy_map)
+        times.append(time.perf_counter() - a)
+    t2 = time.perf_counter()
+    mgr.allocate_cache_if_needed(2 * n)
+    t3 = time.perf_counter()
+    assert mgr.get_key_cache(0) == first_ptr
+    ms = float(np.median(times[1:])) * 1e3
+    moved = 2.0 * blocks * bb  # read + written
+    return {"layers": layers, "blocks_copied": blocks, "copy_blocks_ms": round(ms, 4),
+            "copy_blocks_GBps": round(moved / (ms * 1e-3) / 1e9, 1),
+            "roofline": {"bound": "hbm", "kernel": "kv_copy_blocks_kernel", "achieved": round(moved / (ms * 1e-3) / 1e9, 1),
+                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+            "first_allocation_ms": round((t1 - t0) * 1e3, 3), "growth_to_twice_ms": round((t3 - t2) * 1e3, 3),
+            "cache_bytes_after_growth": 2 * n * bb,
+            "note": "copy: one upload of the pair list, one launch over (pair, layer, K|V), one stream wait; bytes = "
+                    "blocks x block bytes over all layers, read + written.  Growth maps new memory behind the tensors' "
+                    "fixed base addresses and clears it; nothing is copied"}
 
 
 def diversity_leg(torch, op, spec, kc, dev, ev, reps=20):
@@ -441,6 +477,8 @@ def main():
         res["xattention"] = xattention_leg(torch, pkg, dev, args.xattention, "u8" if args.kv_dtype == "u8" else "bf16")
     if args.diversity > 0:
         res["adaptive_rkv_diversity"] = diversity_leg(torch, op, spec, kc, dev, args.diversity)
+    if args.kv_cache_leg:
+        res["kv_cache"] = kv_cache_leg(torch, pkg, dev)
     if args.config == 4:
         res["eviction"] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers)
     if not args.no_cpu_baseline:

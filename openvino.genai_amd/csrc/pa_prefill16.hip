@@ -95,11 +95,10 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 }
 
 // ---- KV block fetches -------------------------------------------------------------------------------------
-// The loads are written as asm and waited for with explicit counts: three blocks stay in flight per thread, and
-// the compiler's own bookkeeping would wait for all of them (vmcnt 0) at every use of the oldest one.  Rules that
-// keep this sound: every step issues exactly LOADS loads per thread (tile indices are clamped rather than
-// skipped), loads return in order, a set is read only after kv_wait on it, and all loads are drained before the
-// registers can be given to anything else.
+// Through registers (u8 caches, whose rows are transformed on the way to LDS; block-sparse items; head size 64):
+// ordinary loads into three register sets, three blocks in flight per thread; the compiler counts the outstanding
+// loads itself (it waits for the oldest set only).  Every step issues the same loads per thread: tile indices are
+// clamped rather than skipped.
 typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 template <bool U8>
 struct KvRegs;
@@ -114,23 +113,38 @@ struct KvRegs<true> {
     u2v kc, kh, vc, vh;  // 8 codes and the row header (scale, zero-point) of a K row and of a V row
 };
 __device__ __forceinline__ void kv_issue(KvRegs<false>& r, const uint8_t* kp, const uint8_t* vp) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.k) : "v"(kp));
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.v) : "v"(vp));
+    r.k = *reinterpret_cast<const u4v*>(kp);
+    r.v = *reinterpret_cast<const u4v*>(vp);
 }
 __device__ __forceinline__ void kv_issue(KvRegs<true>& r, const uint8_t* krow, const uint8_t* vrow, int code_off) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r.kc) : "v"(krow + code_off));
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r.kh) : "v"(krow));
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r.vc) : "v"(vrow + code_off));
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r.vh) : "v"(vrow));
+    r.kc = *reinterpret_cast<const u2v*>(krow + code_off);
+    r.kh = *reinterpret_cast<const u2v*>(krow);
+    r.vc = *reinterpret_cast<const u2v*>(vrow + code_off);
+    r.vh = *reinterpret_cast<const u2v*>(vrow);
 }
-// waits until at most N of this thread's loads are outstanding; the set's registers are valid afterwards
-template <int N>
-__device__ __forceinline__ void kv_wait(KvRegs<false>& r) {
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r.k), "+v"(r.v) : "n"(N));
+
+// Straight into LDS (dense items over 16-bit caches, head size 128): one instruction moves 64 x 16 bytes from
+// per-lane global addresses to 1024 consecutive bytes of LDS at a wave-uniform address; no registers, no LDS stores.
+__device__ __forceinline__ void dma16(const uint8_t* src, uint8_t* lds_dst) {
+    typedef __attribute__((address_space(3))) void* lds_p;
+    typedef const __attribute__((address_space(1))) void* glb_p;
+    __builtin_amdgcn_global_load_lds((glb_p)src, (lds_p)lds_dst, 16, 0, 0);
+}
+// Waits until at most N of the wave's vector-memory operations are outstanding (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14; the other counters left at their maxima).
+// Workgroup barrier for LDS traffic only.  __syncthreads() (and a workgroup fence of any kind) makes the compiler wait
+// for every copy into LDS that is in flight, the prefetched blocks included; here the wave waits for its own LDS
+// operations, meets the others, and the copies it must have finished are named by the caller (wait_vmem).  The
+// barrier instruction and the empty asm statements keep the compiler from moving LDS accesses across.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); vmcnt and expcnt at their maxima
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 template <int N>
-__device__ __forceinline__ void kv_wait(KvRegs<true>& r) {
-    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r.kc), "+v"(r.kh), "+v"(r.vc), "+v"(r.vh) : "n"(N));
+__device__ __forceinline__ void wait_vmem() {
+    __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | 0x0f70);
 }
 
 // DT: type of the MFMA operands and of the rows staged in LDS; QDT: type of query and output; U8: the cache holds
@@ -142,28 +156,44 @@ __device__ __forceinline__ void kv_wait(KvRegs<true>& r) {
 // path needs more registers and stays at two).
 // XATT: the work items belong to block-sparse sequences (never together with PIPE: passing over a block would have
 // to be threaded through three pipeline stages).
-template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT>
-__global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel(PrefillArgs a) {
+// DMA: 256-thread workgroups whose KV blocks go straight from global memory into LDS (four K and four V slots, three
+// blocks in flight behind the one being worked on).  Rows sit in LDS unpadded; instead the 16-byte pieces of row r are
+// stored at piece position p ^ (r & 15), which keeps both operand reads free of bank conflicts -- the permutation is
+// applied on the global side of the copy, each lane fetching the piece that belongs at its LDS position.  With no
+// staging registers the kernel fits three waves per SIMD at two 16-row groups per wave: half the LDS operand traffic
+// per matrix instruction of the one-group variant.
+template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT, bool DMA>
+__global__ __launch_bounds__(DMA ? 256 : 512, DMA ? 2 : (PIPE || U8) ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
+void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     static_assert(!XATT || !PIPE, "the block-sparse variant works a block through in one go");
     static_assert(U8 || DT == QDT, "16-bit caches are used in the query's type");
-    constexpr int NT = 512;
+    static_assert(!DMA || (!U8 && !PIPE && !XATT && D == 128), "the straight-to-LDS variant: dense items, 16-bit caches, head size 128");
+    constexpr int NT = DMA ? 256 : 512;
     constexpr int ROWB = D * 2;            // bytes of a row as staged in LDS
     constexpr int CROWB = U8 ? D + 8 : D * 2;  // bytes of a row in the cache
-    constexpr int LROWK = ROWB + 16;       // LDS row strides chosen so that the operand reads are bank-conflict free:
-    constexpr int LROWV = ROWB + 32;       // K rows are read 16 B per lane, V rows 32 B per 4 lanes (transpose read)
+    constexpr int LROWK = DMA ? ROWB : ROWB + 16;  // LDS row strides chosen so that the operand reads are bank-conflict free:
+    constexpr int LROWV = DMA ? ROWB : ROWB + 32;  // K rows are read 16 B per lane, V rows 32 B per 4 lanes (transpose read)
     constexpr int TILEK = TOK * LROWK, TILEV = TOK * LROWV;
+    constexpr int NKS = DMA ? 4 : 2, NVS = 4;  // K and V slots
     constexpr int KS = D / 32;
     constexpr int RT = D / 16;
     constexpr int CPR = ROWB / 16;         // 16-byte chunks per row
     constexpr int NCH = TOK * CPR;         // chunks per block and tensor: 512 (D = 128) or 256 (D = 64)
-    static_assert(NCH <= NT, "one chunk per thread");
+    static_assert(DMA || NCH <= NT, "one chunk per thread");
     constexpr int HDRB = U8 ? 4 * TOK * 4 : 0;  // per buffer: sc_k | zp_k * sc_k | sc_v | zp_v, one f32 per token each
     constexpr float CODE_UNIT = 16777216.0f;    // a code byte read as f16 is code * 2^-24
     // The loop works on three blocks at once (see the pipeline below): K of block t+1, V of block t-1 and the
     // headers of block t are read while block t+2 is written, hence two K slots and four V / header slots.
-    constexpr int OFF_V = 2 * TILEK, OFF_H = 2 * TILEK + 4 * TILEV;
-    __shared__ __align__(16) uint8_t smem[2 * TILEK + 4 * TILEV + 4 * HDRB];  // K[2] | V[4] | headers[4]
+    constexpr int OFF_V = NKS * TILEK, OFF_H = NKS * TILEK + NVS * TILEV;
+    __shared__ __align__(16) uint8_t smem[DMA ? 16 : NKS * TILEK + NVS * TILEV + 4 * HDRB];  // K slots | V slots | headers[4]
+    // DMA: every slot is an LDS object of its own, so that the compiler can tell a copy into one slot from the operand
+    // reads of another (it orders reads after the copies that may have written what they read; with one array for all
+    // slots that would be every copy in flight, the prefetched blocks included)
+    __shared__ __align__(16) uint8_t dk0[DMA ? TILEK : 16], dk1[DMA ? TILEK : 16], dk2[DMA ? TILEK : 16], dk3[DMA ? TILEK : 16];
+    __shared__ __align__(16) uint8_t dv0[DMA ? TILEV : 16], dv1[DMA ? TILEV : 16], dv2[DMA ? TILEV : 16], dv3[DMA ? TILEV : 16];
+    auto kslot = [](int j) { return (j & 1); };
+    auto vslot = [](int j) { return (j & 3); };
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -299,12 +329,11 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
     // by the causal select, their V rows are cleared here so that 0 * garbage cannot reach the accumulators
     // j = block number within the item's range; it selects the LDS slots
     auto stash = [&](KvRegs<U8>& r, int j) __attribute__((always_inline)) {
-        kv_wait<2 * KvRegs<U8>::LOADS>(r);  // the two younger sets may still be in flight
         const int tile = tile_at(j);
         if (loader && j < cnt) {
             const bool live = tile * TOK + ltid / CPR < kv_len;
-            uint8_t* kd = smem + (j & 1) * TILEK + lds_k;
-            uint8_t* vd = smem + (j & 3) * TILEV + lds_v;
+            uint8_t* kd = smem + kslot(j) * TILEK + lds_k;
+            uint8_t* vd = smem + vslot(j) * TILEV + lds_v;
             if constexpr (U8) {
                 // Codes go to LDS as 16-bit words holding (code - c) * 2^-24, c the integer nearest the row's
                 // zero-point: an exact f16 subnormal either way, but the sums the matrix pipe forms stay near the
@@ -356,15 +385,14 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
     // V operands come through the LDS transpose read: source lane (e = n >> 2, q = n & 3) of a 16-lane group
     // supplies 4 channels of token 16 h + 4 g + e; lane n receives channel 16 r + n of tokens 16 h + 4 g + 0..3.
     auto load_v = [&](const uint8_t* vb, int r) __attribute__((always_inline)) {
-        const uint8_t* p0 = vb + (4 * g + (n >> 2)) * LROWV + (16 * r + 4 * (n & 3)) * 2;
+        const uint8_t* p0 = DMA ? vb + (4 * g + (n >> 2)) * LROWV + (((2 * r + ((n & 3) >> 1)) ^ (4 * g + (n >> 2))) << 4) + 8 * (n & 1)
+                                : vb + (4 * g + (n >> 2)) * LROWV + (16 * r + 4 * (n & 3)) * 2;
         const s4v v0 = lds_read_tr16(p0);
         const s4v v1 = lds_read_tr16(p0 + 16 * LROWV);
         return s8v{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
     };
-    auto qk_pv = [&](bool do_qk, int jk, f4 (&sc)[2][2], bool do_pv, int jv, const u4v (&pb)[2], const u4v (&pl)[2])
-                     __attribute__((always_inline)) {
-        const uint8_t* kb = smem + (jk & 1) * TILEK;
-        const uint8_t* vb = smem + OFF_V + (jv & 3) * TILEV;
+    auto qk_pv_at = [&](bool do_qk, const uint8_t* kb, f4 (&sc)[2][2], bool do_pv, const uint8_t* vb, const u4v (&pb)[2],
+                        const u4v (&pl)[2]) __attribute__((always_inline)) {
         if (do_qk) {
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi) sc[gi][0] = sc[gi][1] = f4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -375,7 +403,8 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
             if (do_qk && s < KS) {
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    const s8v kop = *reinterpret_cast<const s8v*>(kb + (16 * u + n) * LROWK + (32 * s + 8 * g) * 2);
+                    const s8v kop = DMA ? *reinterpret_cast<const s8v*>(kb + (16 * u + n) * LROWK + (((4 * s + g) ^ n) << 4))
+                                        : *reinterpret_cast<const s8v*>(kb + (16 * u + n) * LROWK + (32 * s + 8 * g) * 2);
 #pragma unroll
                     for (int gi = 0; gi < NG; ++gi) sc[gi][u] = mma<DT>(kop, qreg[gi][s], sc[gi][u]);
                 }
@@ -404,6 +433,10 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
                 vprev[1] = vcur[1];
             }
         }
+    };
+    auto qk_pv = [&](bool do_qk, int jk, f4 (&sc)[2][2], bool do_pv, int jv, const u4v (&pb)[2], const u4v (&pl)[2])
+                     __attribute__((always_inline)) {
+        qk_pv_at(do_qk, smem + kslot(jk) * TILEK, sc, do_pv, smem + OFF_V + vslot(jv) * TILEV, pb, pl);
     };
     // masks + online softmax of block `tile` (number j): probabilities as MFMA operands, rescale factors.
     // The running maximum is only raised when a block exceeds it by more than 2^4: probabilities then stay
@@ -548,11 +581,12 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
     };
 
     // without the pipeline: block number j start to end (QK, softmax, rescale, PV)
-    auto body_whole = [&](auto masked_c, int j, const bool (&kept)[2]) __attribute__((always_inline)) {
+    auto body_whole = [&](auto masked_c, int j, const bool (&kept)[2], const uint8_t* kb, const uint8_t* vb)
+                          __attribute__((always_inline)) {
         f4 sc[2][2];
         u4v pb[2], pl[2];
         float corr[2];
-        qk_pv(true, j, sc, false, 0, pb, pl);
+        qk_pv_at(true, kb, sc, false, vb, pb, pl);
         softmax(masked_c, sc, tile_at(j), j, pb, pl, corr, kept);
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi) {
@@ -561,9 +595,9 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
                 for (int r = 0; r < RT; ++r) acc[gi][r] *= corr[gi];
             }
         }
-        qk_pv(false, 0, sc, true, j, pb, pl);
+        qk_pv_at(false, kb, sc, true, vb, pb, pl);
     };
-    auto whole = [&](int j) __attribute__((always_inline)) {
+    auto whole_at = [&](int j, const uint8_t* kb, const uint8_t* vb) __attribute__((always_inline)) {
         const int tile = tile_at(j);
         bool kept[2] = {true, true};
         if constexpr (XATT) {
@@ -574,61 +608,114 @@ __global__ __launch_bounds__(512, (PIPE || U8) ? 2 : 4) void pa_prefill16_kernel
             }
         }
         if (XATT || tile * TOK < free_lo || tile * TOK + TOK - 1 > free_hi)  // wave-uniform
-            body_whole(std::true_type{}, j, kept);
+            body_whole(std::true_type{}, j, kept, kb, vb);
         else
-            body_whole(std::false_type{}, j, kept);
+            body_whole(std::false_type{}, j, kept, kb, vb);
+    };
+    auto whole = [&](int j) __attribute__((always_inline)) {
+        whole_at(j, smem + kslot(j) * TILEK, smem + OFF_V + vslot(j) * TILEV);
     };
 
-    fetch(set[0], 0);
-    fetch(set[1], 1);
-    fetch(set[2], 2);
-    // step 0 multiplies V slot 3 by zero probabilities: make sure it holds numbers
-    if (loader) *reinterpret_cast<u4v*>(smem + 3 * TILEV + lds_v) = u4v{0u, 0u, 0u, 0u};
-    // the query loads (issued above, tracked by the compiler) are waited for here, not inside the loop
+    if constexpr (DMA) {
+        // Block number j lives in K slot and V slot j % 4.  A wave moves rows 8 wv .. 8 wv + 7 of a block: lane l of
+        // its two instructions per tensor takes row 8 wv + 4 i + l / 16, LDS piece position l % 16, i.e. the row's
+        // piece (l % 16) ^ (row & 15).  Every step issues the same four copies per wave (indices clamped), so that
+        // "at most eight outstanding" always means: everything but the two youngest blocks has landed.
+        const int my_row = 8 * wv + (lane >> 4);          // + 4 for the second instruction
+        const int my_piece = ((lane & 15) ^ (my_row & 15)) << 4;
+        const int my_piece2 = ((lane & 15) ^ ((my_row + 4) & 15)) << 4;
+        auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
+            const long blk = ((long)table[tile_at(j)] * Hkv + hkv) * (TOK * CROWB);
+            const uint8_t* kg = a.key_cache + blk + my_row * ROWB;
+            const uint8_t* vg = a.value_cache + blk + my_row * ROWB;
+            uint8_t* kd = kslot_base + wv * 2048;
+            uint8_t* vd = vslot_base + wv * 2048;
+            dma16(kg + my_piece, kd);
+            dma16(kg + 4 * ROWB + my_piece2, kd + 1024);
+            dma16(vg + my_piece, vd);
+            dma16(vg + 4 * ROWB + my_piece2, vd + 1024);
+        };
+        copy_in(0, dk0, dv0);
+        copy_in(1, dk1, dv1);
+        copy_in(2, dk2, dv2);
+        // the query loads (issued above, tracked by the compiler) are waited for here, not inside the loop
 #pragma unroll
-    for (int gi = 0; gi < NG; ++gi)
+        for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
-        for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qreg[gi][s]));
-    stash(set[0], 0);
-    fetch(set[0], 3);
-    stash(set[1], 1);
-    __syncthreads();
-    if (active) {
-        if (PIPE)
-            qk_pv(true, 0, s_cur, false, 0, pb_prev, pl_prev);
-        else if (cnt > 0)  // a block-sparse item may have nothing left to do
-            whole(0);
+            for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qreg[gi][s]));
+        // step j: block j sits in slot j % 4 (kc, vc); the slot of block j - 1 (kn, vn) takes block j + 3
+#define PA_DMA_STEP(kc, vc, kn, vn)                                                                      \
+        {                                                                                                \
+            if (j >= cnt) break;                                                                         \
+            wait_vmem<8>();  /* this wave's part of block j has landed (blocks j + 1, j + 2 may be on their way) */ \
+            lds_barrier();   /* so has everyone else's, and block j - 1 is done with */                  \
+            copy_in(j + 3, kn, vn);                                                                      \
+            const int tile = tile_at(j);                                                                 \
+            if (tile * TOK + TOK > kv_len) { /* (uniform) the sequence's last block: clear the V rows beyond its tokens */ \
+                for (int c = tid; c < (TOK - (kv_len - tile * TOK)) * CPR; c += NT)                       \
+                    *reinterpret_cast<u4v*>(vc + (kv_len - tile * TOK) * LROWV + c * 16) = u4v{0u, 0u, 0u, 0u}; \
+                lds_barrier();                                                                           \
+            }                                                                                            \
+            if (active) whole_at(j, kc, vc);                                                             \
+            ++j;                                                                                         \
+        }
+        for (int j = 0;;) {
+            PA_DMA_STEP(dk0, dv0, dk3, dv3)
+            PA_DMA_STEP(dk1, dv1, dk0, dv0)
+            PA_DMA_STEP(dk2, dv2, dk1, dv1)
+            PA_DMA_STEP(dk3, dv3, dk2, dv2)
+        }
+#undef PA_DMA_STEP
+        wait_vmem<0>();  // the clamped copies of the last three steps still target this workgroup's LDS
+    } else {
+        fetch(set[0], 0);
+        fetch(set[1], 1);
+        fetch(set[2], 2);
+        // step 0 multiplies V slot 3 by zero probabilities: make sure it holds numbers
+        if (loader) *reinterpret_cast<u4v*>(smem + 3 * TILEV + lds_v) = u4v{0u, 0u, 0u, 0u};
+        // the query loads (issued above, tracked by the compiler) are waited for here, not inside the loop
+    #pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+    #pragma unroll
+            for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qreg[gi][s]));
+        stash(set[0], 0);
+        fetch(set[0], 3);
+        stash(set[1], 1);
+        __syncthreads();
+        if (active) {
+            if (PIPE)
+                qk_pv(true, 0, s_cur, false, 0, pb_prev, pl_prev);
+            else if (cnt > 0)  // a block-sparse item may have nothing left to do
+                whole(0);
+        }
+        __syncthreads();  // step 0 overwrites K slot 0, which the lines above read
+        // step j: set (j+1)%3 was written to LDS in step j-1 and takes block t+4; set (j+2)%3 holds block t+2.
+        // Without the pipeline step j works on block t+1 (whose K and V are both in LDS by then); block tb was done above.
+    #define PA_STEP(K)                                                                       \
+        {                                                                                    \
+            const int j = i + K, tile = tb + j; /* PIPE is never block-sparse */           \
+            if (j >= cnt) break;                                                             \
+            fetch(set[(K + 1) % 3], j + 4);                                                  \
+            if (active) {                                                                    \
+                if (!PIPE) {                                                                 \
+                    if (j + 1 < cnt) whole(j + 1);                                           \
+                } else if (tile * TOK < free_lo || tile * TOK + TOK - 1 > free_hi) { /* wave-uniform */ \
+                    body(std::true_type{}, j);                                               \
+                } else {                                                                     \
+                    body(std::false_type{}, j);                                              \
+                }                                                                            \
+            }                                                                                \
+            stash(set[(K + 2) % 3], j + 2);                                                  \
+            __syncthreads();                                                                 \
+        }
+        for (int i = 0;; i += 3) {
+            PA_STEP(0)
+            PA_STEP(1)
+            PA_STEP(2)
+        }
+    #undef PA_STEP
     }
-    __syncthreads();  // step 0 overwrites K slot 0, which the lines above read
-    // step j: set (j+1)%3 was written to LDS in step j-1 and takes block t+4; set (j+2)%3 holds block t+2.
-    // Without the pipeline step j works on block t+1 (whose K and V are both in LDS by then); block tb was done above.
-#define PA_STEP(K)                                                                       \
-    {                                                                                    \
-        const int j = i + K, tile = tb + j; /* PIPE is never block-sparse */           \
-        if (j >= cnt) break;                                                             \
-        fetch(set[(K + 1) % 3], j + 4);                                                  \
-        if (active) {                                                                    \
-            if (!PIPE) {                                                                 \
-                if (j + 1 < cnt) whole(j + 1);                                           \
-            } else if (tile * TOK < free_lo || tile * TOK + TOK - 1 > free_hi) { /* wave-uniform */ \
-                body(std::true_type{}, j);                                               \
-            } else {                                                                     \
-                body(std::false_type{}, j);                                              \
-            }                                                                            \
-        }                                                                                \
-        stash(set[(K + 2) % 3], j + 2);                                                  \
-        __syncthreads();                                                                 \
-    }
-    for (int i = 0;; i += 3) {
-        PA_STEP(0)
-        PA_STEP(1)
-        PA_STEP(2)
-    }
-#undef PA_STEP
     if (PIPE && active) qk_pv(false, 0, s_cur, true, te - 1 - tb, pb_prev, pl_prev);  // the last block's V
-    kv_wait<0>(set[0]);  // drain the clamped tail fetches before their registers are reused
-    kv_wait<0>(set[1]);
-    kv_wait<0>(set[2]);
 
     // ---- write the rows ------------------------------------------------------------------------------
     const bool final_out = item.nsplit == 1;
@@ -744,14 +831,24 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
     if (a.n_wide > 0) {  // items with more than 16 query rows
         PrefillArgs w = a;
         w.n_items = a.n_wide;
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, true, false>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(512), 0, s, w);
+        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, true, false, false>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(512), 0, s, w);
     }
     const int n_narrow = a.n_items - a.n_sparse - a.n_wide - (a.skip_single ? a.n_single : 0);
     if (n_narrow > 0) {  // the rest of the dense ones, listed behind them
         PrefillArgs nrw = a;
         nrw.items = a.items + a.n_wide;
         nrw.n_items = n_narrow;
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, false>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(512), 0, s, nrw);
+        // 16-bit caches, head size 128, chunks only: blocks straight into LDS, two row groups per wave.  (Items of
+        // single-token sequences hold a handful of rows: next to them the one-group variant, with more waves moving
+        // blocks and half the arithmetic on empty rows, is the faster one -- 0.25 against 0.31 ms on the mixed workload.)
+        bool straight = false;
+        if constexpr (!U8 && D == 128) straight = a.n_single == 0 || a.skip_single;
+        if constexpr (!U8 && D == 128) {
+            if (straight)
+                hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, false, true>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(256), 0, s, nrw);
+        }
+        if (!straight)
+            hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, false, false>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(512), 0, s, nrw);
     }
     if (a.n_sparse > 0) {  // the items of block-sparse sequences come last
         PrefillArgs sp = a;
@@ -759,7 +856,7 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
         sp.n_items = a.n_sparse;
         // 128 query rows per workgroup whatever the cache: the fewer tokens share a work item, the fewer KV blocks
         // it has to walk for rows that did not keep them
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, true>), dim3((unsigned)sp.n_items * a.sh.Hkv), dim3(512), 0, s, sp);
+        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, true, false>), dim3((unsigned)sp.n_items * a.sh.Hkv), dim3(512), 0, s, sp);
     }
     if (ev1) (void)hipEventRecord(ev1, s);
     if (a.n_merge > 0) {

@@ -598,6 +598,25 @@ pa_evictor* make(const pa_evictor_config* cfg, bool areas, uint64_t ignore_block
     }
     ev->slot_mark.assign(cfg->max_sequences, 0);
     const size_t pairs = (size_t)cfg->max_sequences * cfg->num_decoder_layers;
+    try {  // what a call over every slot uploads and reads back at least, so that the first call does not allocate it
+        const size_t up = ((size_t)cfg->num_decoder_layers * sizeof(float*) + 15) / 16 * 16 + pairs * sizeof(RegEntry);
+        ev->h_up.reserve(up);
+        ev->d_entries.reserve(pairs * std::max(sizeof(RegEntry), sizeof(SelEntry)));
+        ev->d_ptrs.reserve((size_t)cfg->num_decoder_layers * sizeof(float*));
+        ev->d_list.reserve(pairs * sizeof(int32_t));
+        ev->h_back.reserve(pairs * sizeof(int32_t));
+    } catch (...) {
+        (void)hipFree(ev->scores);
+        (void)hipFree(ev->counters);
+        if (ev->hist) (void)hipFree(ev->hist);
+        ev->h_up.release();
+        ev->d_entries.release();
+        ev->d_ptrs.release();
+        ev->d_list.release();
+        (void)hipEventDestroy(ev->staged);
+        delete ev;
+        throw;
+    }
     ev->len.assign(pairs, 0);
     ev->snapkv_seen.assign(cfg->max_sequences, 0);
     if (ev->rkv()) {

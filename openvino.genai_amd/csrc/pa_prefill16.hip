@@ -157,9 +157,11 @@ __device__ __forceinline__ void wait_vmem() {
 // XATT: the work items belong to block-sparse sequences (never together with PIPE: passing over a block would have
 // to be threaded through three pipeline stages).
 // DMA: 256-thread workgroups whose KV blocks go straight from global memory into LDS (four K and four V slots, three
-// blocks in flight behind the one being worked on).  Rows sit in LDS unpadded; instead the 16-byte pieces of row r are
-// stored at piece position p ^ (r & 15), which keeps both operand reads free of bank conflicts -- the permutation is
-// applied on the global side of the copy, each lane fetching the piece that belongs at its LDS position.  With no
+// blocks in flight behind the one being worked on).  Rows sit in LDS unpadded; instead the 16-byte pieces of a row are
+// permuted: K row r keeps piece p at position p ^ (r & 15) (16 lanes read one piece of 16 rows), V row r at
+// p ^ 2 (r & 7) (the transpose read takes 32 bytes of each of four consecutive rows), which keeps both operand reads
+// free of bank conflicts -- the permutation is applied on the global side of the copy, each lane fetching the piece
+// that belongs at its LDS position.  With no
 // staging registers the kernel fits three waves per SIMD at two 16-row groups per wave: half the LDS operand traffic
 // per matrix instruction of the one-group variant.
 template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT, bool DMA>
@@ -385,7 +387,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
     // V operands come through the LDS transpose read: source lane (e = n >> 2, q = n & 3) of a 16-lane group
     // supplies 4 channels of token 16 h + 4 g + e; lane n receives channel 16 r + n of tokens 16 h + 4 g + 0..3.
     auto load_v = [&](const uint8_t* vb, int r) __attribute__((always_inline)) {
-        const uint8_t* p0 = DMA ? vb + (4 * g + (n >> 2)) * LROWV + (((2 * r + ((n & 3) >> 1)) ^ (4 * g + (n >> 2))) << 4) + 8 * (n & 1)
+        const uint8_t* p0 = DMA ? vb + (4 * g + (n >> 2)) * LROWV + (((2 * r + ((n & 3) >> 1)) ^ (((4 * g + (n >> 2)) & 7) << 1)) << 4) + 8 * (n & 1)
                                 : vb + (4 * g + (n >> 2)) * LROWV + (16 * r + 4 * (n & 3)) * 2;
         const s4v v0 = lds_read_tr16(p0);
         const s4v v1 = lds_read_tr16(p0 + 16 * LROWV);
@@ -624,6 +626,8 @@ void pa_prefill16_kernel(PrefillArgs a) {
         const int my_row = 8 * wv + (lane >> 4);          // + 4 for the second instruction
         const int my_piece = ((lane & 15) ^ (my_row & 15)) << 4;
         const int my_piece2 = ((lane & 15) ^ ((my_row + 4) & 15)) << 4;
+        const int my_vpiece = ((lane & 15) ^ ((my_row & 7) << 1)) << 4;
+        const int my_vpiece2 = ((lane & 15) ^ (((my_row + 4) & 7) << 1)) << 4;
         auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
             const long blk = ((long)table[tile_at(j)] * Hkv + hkv) * (TOK * CROWB);
             const uint8_t* kg = a.key_cache + blk + my_row * ROWB;
@@ -632,8 +636,8 @@ void pa_prefill16_kernel(PrefillArgs a) {
             uint8_t* vd = vslot_base + wv * 2048;
             dma16(kg + my_piece, kd);
             dma16(kg + 4 * ROWB + my_piece2, kd + 1024);
-            dma16(vg + my_piece, vd);
-            dma16(vg + 4 * ROWB + my_piece2, vd + 1024);
+            dma16(vg + my_vpiece, vd);
+            dma16(vg + 4 * ROWB + my_vpiece2, vd + 1024);
         };
         copy_in(0, dk0, dv0);
         copy_in(1, dk1, dv1);

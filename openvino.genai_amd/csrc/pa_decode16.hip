@@ -66,9 +66,10 @@ __device__ __forceinline__ float group_sum(float v) {
     return v + __shfl_xor(v, 32, WAVE);
 }
 
-template <int D, int DT>
+template <int D, int DT, int BS>
 __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
     constexpr int WAVES = 4;
+    constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile (with two, each holds one row group)
     constexpr int ROWB = D * 2;            // bytes of a cache row
     constexpr int TILE = TOK * ROWB;       // bytes of one (block, head) of K or V
     constexpr int LROWV = ROWB + 32;       // LDS row stride of the V slot (the transposing reads are conflict free)
@@ -107,22 +108,27 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
         u4v k[2][KS];
         u4v v[VCH];
     };
-    auto issue = [&](Block& blk, int phys) __attribute__((always_inline)) {
-        const long base = ((long)phys * Hkv + hkv) * TILE;
-        const uint8_t* kp = a.key_cache + base;
-        const u4v* vp = reinterpret_cast<const u4v*>(a.value_cache + base);
+    // the tile's two row groups: halves of the block `phys0`, or the 16-token blocks `phys0` and `phys1`
+    auto issue = [&](Block& blk, int phys0, int phys1) __attribute__((always_inline)) {
+        const long base0 = ((long)phys0 * Hkv + hkv) * (TILE / BPT);
+        const long base1 = BS == TOK ? base0 + TILE / 2 : ((long)phys1 * Hkv + hkv) * (TILE / 2);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int s = 0; s < KS; ++s)
-                blk.k[u][s] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(kp + (16 * u + n) * ROWB + (32 * s + 8 * g) * 2));
+                blk.k[u][s] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(
+                    a.key_cache + (u ? base1 : base0) + n * ROWB + (32 * s + 8 * g) * 2));
+        static_assert(VCH % 2 == 0, "each half of the V tile is a whole number of wave passes");
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) blk.v[c] = __builtin_nontemporal_load(vp + c * 64 + lane);
+        for (int c = 0; c < VCH; ++c)
+            blk.v[c] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(
+                           a.value_cache + (c < VCH / 2 ? base0 : base1 - TILE / 2)) + c * 64 + lane);
     };
+    const int last_block = (kv_len + BS - 1) / BS - 1;  // a last tile of one 16-token block repeats it (rows masked)
     Block ba, bb;
     int tile = tb + wv;
-    if (tile < te) issue(ba, table[tile]);
-    for (int i = tid; i < te - tb; i += 64 * WAVES) tab[i] = table[tb + i];
+    if (tile < te) issue(ba, table[min(BPT * tile, last_block)], table[min(BPT * tile + BPT - 1, last_block)]);
+    for (int i = tid; i < BPT * (te - tb); i += 64 * WAVES) tab[i] = table[min(BPT * tb + i, last_block)];
 
     // query operand (B of QK): lane (n, g) holds q[head n][32 s + 8 g + e]; heads beyond the group are zero
     s8v qreg[KS];
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
 
     auto process = [&](Block& cur, Block& nxt, const int tl) __attribute__((always_inline)) {
         // next block's loads into flight, this block's V into the slot
-        if (tl + WAVES < te) issue(nxt, tab[tl + WAVES - tb]);
+        if (tl + WAVES < te) issue(nxt, tab[BPT * (tl + WAVES - tb)], tab[BPT * (tl + WAVES - tb) + BPT - 1]);
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
             const int piece = c * 64 + lane;
@@ -345,13 +351,13 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
     }
 }
 
-template <int D, int DT>
-hipError_t launch_decode16_typed(hipStream_t s, const DecodeArgs& a_in, hipEvent_t ev0, hipEvent_t ev1) {
+template <int D, int DT, int BS>
+hipError_t launch_decode16_sized(hipStream_t s, const DecodeArgs& a_in, hipEvent_t ev0, hipEvent_t ev1) {
     DecodeArgs a = a_in;
     size_t lds = decode16_lds_bytes(D, a.G, a.max_tiles, a.want_scores != 0);
     a.table_off = (int32_t)lds;
-    lds += ((size_t)a.max_tiles * sizeof(int32_t) + 15) & ~(size_t)15;
-    auto kern = pa_decode16_kernel<D, DT>;
+    lds += decode16_table_bytes(a.max_tiles, BS);
+    auto kern = pa_decode16_kernel<D, DT, BS>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     if (ev0) (void)hipEventRecord(ev0, s);
@@ -360,7 +366,16 @@ hipError_t launch_decode16_typed(hipStream_t s, const DecodeArgs& a_in, hipEvent
     return hipGetLastError();
 }
 
+template <int D, int DT>
+hipError_t launch_decode16_typed(hipStream_t s, const DecodeArgs& a, hipEvent_t ev0, hipEvent_t ev1) {
+    return a.sh.bs == 16 ? launch_decode16_sized<D, DT, 16>(s, a, ev0, ev1) : launch_decode16_sized<D, DT, 32>(s, a, ev0, ev1);
+}
+
 }  // namespace
+
+size_t decode16_table_bytes(int max_tiles, int block_size) {
+    return ((size_t)max_tiles * (TOK / block_size) * sizeof(int32_t) + 15) & ~(size_t)15;
+}
 
 // LDS in front of the block-table slice: V slots | per-wave (m, l) | [scores: block maxima | probabilities]
 size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores) {
@@ -371,7 +386,7 @@ size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores) {
 
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,
                            hipEvent_t ev1) {
-    if (a.sh.bs != TOK || a.G > 16 || (a.want_scores != 0) != (scores != nullptr)) return hipErrorInvalidValue;
+    if ((a.sh.bs != 32 && a.sh.bs != 16) || a.G > 16 || (a.want_scores != 0) != (scores != nullptr)) return hipErrorInvalidValue;
     hipError_t e;
     if (a.sh.D == 128) e = dtype == DT_F16 ? launch_decode16_typed<128, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<128, DT_BF16>(s, a, ev0, ev1);
     else if (a.sh.D == 64) e = dtype == DT_F16 ? launch_decode16_typed<64, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<64, DT_BF16>(s, a, ev0, ev1);

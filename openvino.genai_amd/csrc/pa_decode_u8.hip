@@ -68,24 +68,43 @@ __device__ inline float xor_reduce_sum_g(float v) {
     return a + b;
 }
 
-// Loads one block's K and V: whole-wave 16-byte passes plus the 16-chunk tails (K on lanes 0-15, V on 16-31).
-template <int FULL>
-__device__ __forceinline__ void issue_block(const DecodeArgs& a, int phys, int hkv, int tile_bytes, int lane,
+// Loads one 32-token tile of K and V: whole-wave 16-byte passes plus the 16-chunk tails (K on lanes 0-15, V on 16-31).
+// With 32-token cache blocks the tile is the block `phys0`; with 16-token blocks its halves are the blocks `phys0` and
+// `phys1`, and each 16-byte chunk comes from the block its row lies in (the LDS image is the same).
+template <int FULL, int BS>
+__device__ __forceinline__ void issue_block(const DecodeArgs& a, int phys0, int phys1, int hkv, int tile_bytes, int lane,
                                             u4v (&kraw)[FULL], u4v (&vraw)[FULL], u4v& traw) {
-    const long base = ((long)phys * a.sh.Hkv + hkv) * tile_bytes;
-    const u4v* kp = reinterpret_cast<const u4v*>(a.key_cache + base);
-    const u4v* vp = reinterpret_cast<const u4v*>(a.value_cache + base);
+    if (BS == TOK) {
+        const long base = ((long)phys0 * a.sh.Hkv + hkv) * tile_bytes;
+        const u4v* kp = reinterpret_cast<const u4v*>(a.key_cache + base);
+        const u4v* vp = reinterpret_cast<const u4v*>(a.value_cache + base);
 #pragma unroll
-    // every cache byte is used once per launch: streaming (non-temporal) loads keep it from displacing L2 contents
-    for (int c = 0; c < FULL; ++c) {
-        kraw[c] = __builtin_nontemporal_load(kp + c * 64 + lane);
-        vraw[c] = __builtin_nontemporal_load(vp + c * 64 + lane);
+        // every cache byte is used once per launch: streaming (non-temporal) loads keep it from displacing L2 contents
+        for (int c = 0; c < FULL; ++c) {
+            kraw[c] = __builtin_nontemporal_load(kp + c * 64 + lane);
+            vraw[c] = __builtin_nontemporal_load(vp + c * 64 + lane);
+        }
+        traw = __builtin_nontemporal_load(((lane & 16) ? vp : kp) + FULL * 64 + (lane & 15));
+    } else {
+        const int half = tile_bytes / 2, half_chunks = half / 16;  // the tails lie in the second half
+        const long base0 = ((long)phys0 * a.sh.Hkv + hkv) * half;
+        const long base1 = ((long)phys1 * a.sh.Hkv + hkv) * half - half;
+#pragma unroll
+        for (int c = 0; c < FULL; ++c) {
+            const int ci = c * 64 + lane;
+            const long off = (ci < half_chunks ? base0 : base1) + (long)ci * 16;
+            kraw[c] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(a.key_cache + off));
+            vraw[c] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(a.value_cache + off));
+        }
+        const long toff = base1 + (long)(FULL * 64 + (lane & 15)) * 16;
+        traw = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(((lane & 16) ? a.value_cache : a.key_cache) + toff));
     }
-    traw = __builtin_nontemporal_load(((lane & 16) ? vp : kp) + FULL * 64 + (lane & 15));
 }
 
-template <int D, int QDT, int WAVES>
+template <int D, int QDT, int WAVES, int BS>
 __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs a) {
+    constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile
+    static_assert(BS == 32 || (BS == 16 && WAVES == 4), "the descriptor holds the ids of the first eight tiles");
     constexpr int NT = 64 * WAVES;
     constexpr int ROW = D + 8;
     constexpr int TILE = TOK * ROW;        // bytes of one (block, head) of K or V
@@ -129,7 +148,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
     auto append_rows = [&]() __attribute__((always_inline)) {
         const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
-        const long dst = (((long)dsc->last_id * Hkv + hkv) * TOK + (kv_len - 1) % TOK) * ROW;
+        const long dst = (((long)dsc->last_id * Hkv + hkv) * BS + (kv_len - 1) % BS) * ROW;
         uint16_t kr[EPL], vr[EPL];
         load_row16<EPL>(a.key + src, kr);
         load_row16<EPL>(a.value + src, vr);
@@ -144,12 +163,19 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     // the first two blocks' loads go out before anything else is fetched
     u4v kraw[FULL], vraw[FULL], traw, kraw2[FULL], vraw2[FULL], traw2;
     int tile = tb + wv;
-    if (tile < te) issue_block<FULL>(a, dsc->ids[wv], hkv, TILE, lane, kraw, vraw, traw);
-    if (tile + WAVES < te) issue_block<FULL>(a, dsc->ids[wv + WAVES], hkv, TILE, lane, kraw2, vraw2, traw2);
+    if (tile < te)
+        issue_block<FULL, BS>(a, dsc->ids[BPT * wv], dsc->ids[BPT * wv + BPT - 1], hkv, TILE, lane, kraw, vraw, traw);
+    if (tile + WAVES < te)
+        issue_block<FULL, BS>(a, dsc->ids[BPT * (wv + WAVES)], dsc->ids[BPT * (wv + WAVES) + BPT - 1], hkv, TILE, lane, kraw2,
+                              vraw2, traw2);
     if (appends && !append_first) append_rows();
     // this workgroup's slice of the block table, so that no later block fetch waits on a table fetch
     int32_t* tab = reinterpret_cast<int32_t*>(smem + a.table_off);
-    for (int i = tid; i < te - tb; i += NT) tab[i] = table[tb + i];
+    // (16-token blocks: two ids per tile; a last tile of one block repeats it, its second half lies beyond kv_len)
+    {
+        const int last_block = (kv_len + BS - 1) / BS - 1;
+        for (int i = tid; i < BPT * (te - tb); i += NT) tab[i] = table[min(BPT * tb + i, last_block)];
+    }
 
     // query operand (B of QK): lane (n, g) holds q[head n][32 s + 8 g + e]
     h8 qreg[KS];
@@ -223,7 +249,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
 #pragma unroll
         for (int c = 0; c < FULL; ++c) reinterpret_cast<u4v*>(slot)[c * 64 + lane] = vr[c];
         if (lane >= 16 && lane < 32) reinterpret_cast<u4v*>(slot)[FULL * 64 + lane - 16] = tr;
-        if (tile + 2 * WAVES < te) issue_block<FULL>(a, tab[tile + 2 * WAVES - tb], hkv, TILE, lane, kr, vr, tr);
+        if (tile + 2 * WAVES < te) {
+            const int ti = BPT * (tile + 2 * WAVES - tb);
+            issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], hkv, TILE, lane, kr, vr, tr);
+        }
         __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax (log2 domain) -------------------------------------------------------
@@ -627,21 +656,21 @@ __global__ __launch_bounds__(256) void pa_decode_post_kernel(DecodeArgs a, float
 }  // namespace
 
 // LDS layout: staging | per-wave (m, l, z) | [scores: block maxima | probabilities] | block-table slice
-size_t decode_u8_lds_bytes(int D, int G, int max_tiles, bool want_scores, int waves, int32_t* table_off) {
+size_t decode_u8_lds_bytes(int D, int G, int max_tiles, bool want_scores, int waves, int32_t* table_off, int block_size) {
     size_t bytes = (size_t)waves * TOK * (D + 8) + waves * 16 * 4 * sizeof(float);
     if (want_scores) bytes += (size_t)max_tiles * 16 * sizeof(float) + (size_t)G * max_tiles * TOK * sizeof(uint16_t);
     bytes = (bytes + 15) & ~(size_t)15;
     *table_off = (int32_t)bytes;
-    bytes += (size_t)max_tiles * sizeof(int32_t);
+    bytes += (size_t)max_tiles * (TOK / block_size) * sizeof(int32_t);
     return (bytes + 15) & ~(size_t)15;
 }
 
-template <int D, int QDT, int WAVES>
+template <int D, int QDT, int WAVES, int BS>
 static hipError_t launch_decode_typed(hipStream_t s, const DecodeArgs& a_in, float* scores, int max_kv_len,
                                       hipEvent_t ev0, hipEvent_t ev1) {
     DecodeArgs a = a_in;
-    const size_t lds = decode_u8_lds_bytes(D, a.G, a.max_tiles, a.want_scores != 0, WAVES, &a.table_off);
-    auto kern = pa_decode_u8_kernel<D, QDT, WAVES>;
+    const size_t lds = decode_u8_lds_bytes(D, a.G, a.max_tiles, a.want_scores != 0, WAVES, &a.table_off, BS);
+    auto kern = pa_decode_u8_kernel<D, QDT, WAVES, BS>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     if (a.n_seqs > 65535) return hipErrorInvalidValue;  // grid z
@@ -654,8 +683,13 @@ static hipError_t launch_decode_typed(hipStream_t s, const DecodeArgs& a_in, flo
 template <int D, int QDT>
 static hipError_t launch_decode_waves(hipStream_t s, const DecodeArgs& a, float* scores, int max_kv_len,
                                       hipEvent_t ev0, hipEvent_t ev1) {
-    if (a.waves == 8) return launch_decode_typed<D, QDT, 8>(s, a, scores, max_kv_len, ev0, ev1);
-    return launch_decode_typed<D, QDT, 4>(s, a, scores, max_kv_len, ev0, ev1);
+    if (a.sh.bs == 16) {
+        if (a.waves != 4) return hipErrorInvalidValue;
+        return launch_decode_typed<D, QDT, 4, 16>(s, a, scores, max_kv_len, ev0, ev1);
+    }
+    if (a.sh.bs != 32) return hipErrorInvalidValue;
+    if (a.waves == 8) return launch_decode_typed<D, QDT, 8, 32>(s, a, scores, max_kv_len, ev0, ev1);
+    return launch_decode_typed<D, QDT, 4, 32>(s, a, scores, max_kv_len, ev0, ev1);
 }
 
 hipError_t launch_decode_scores(hipStream_t s, const DecodeArgs& a, float* scores, int max_kv_len) {

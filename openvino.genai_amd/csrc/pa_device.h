@@ -193,7 +193,7 @@ struct DecodeArgs {
 __host__ __device__ inline long p_split_offset(long score_offset, int b) { return ((score_offset + 7) & ~7L) + 8L * b; }
 __host__ __device__ inline long p_split_stride(long total_scores, int B) { return total_scores + 8L * B + 8; }
 
-size_t decode_u8_lds_bytes(int D, int G, int max_tiles, bool want_scores, int waves, int32_t* table_off);
+size_t decode_u8_lds_bytes(int D, int G, int max_tiles, bool want_scores, int waves, int32_t* table_off, int block_size);
 // ev0 / ev1 (may be null) are recorded right before and after the main kernel.
 hipError_t launch_decode_u8(hipStream_t s, const DecodeArgs& a, int q_dtype, float* scores, int max_kv_len,
                             hipEvent_t ev0, hipEvent_t ev1);
@@ -228,6 +228,7 @@ struct XattDev {            // what the attention and score kernels need of it (
 // The 16-bit-cache decode kernel (pa_decode16.hip): takes the arguments of the u8 family and leaves split partials,
 // per-kv-head score sums and split probabilities in its layouts (table_off is set by the launcher).
 size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores);
+size_t decode16_table_bytes(int max_tiles, int block_size);  // the block-table slice behind it
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,
                            hipEvent_t ev1);
 // The merge and score kernels of the decode family on their own.

@@ -238,6 +238,8 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
             const int32_t lo = first / 32, hi = (kv_len + 31) / 32;
             const int32_t per = (hi - lo + nsplit - 1) / nsplit;
             const int32_t* tab = ids + ctx->h_bib[b];
+            // cache blocks per 32-token tile, and the sequence's last block (a last tile of one 16-token block repeats it)
+            const int32_t bpt = 32 / ctx->cfg.block_size, last_block = (kv_len - 1) / ctx->cfg.block_size;
             for (int32_t s = 0; s < nsplit; ++s) {
                 pa::DecodeDesc& d = out[i * nsplit + s];
                 d.b = b;
@@ -248,8 +250,9 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
                 d.te = std::min(hi, d.tb + per);
                 d.table_off = ctx->h_bib[b];
                 d.score_off = soff[b];
-                d.last_id = tab[hi - 1];
-                for (int32_t j = 0; j < 16; ++j) d.ids[j] = d.tb + j < d.te ? tab[d.tb + j] : 0;
+                d.last_id = tab[last_block];
+                for (int32_t j = 0; j < 16; ++j)
+                    d.ids[j] = bpt * d.tb + j < bpt * d.te ? tab[std::min(bpt * d.tb + j, last_block)] : 0;
             }
         }
     }
@@ -262,10 +265,13 @@ void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
                                    ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
 }
 
-// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).
+// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).  Its tiles are 32
+// tokens: one 32-token cache block or two 16-token ones.  The matrix kernel that takes the other sequences of a step
+// is built for 32-token blocks only, so with 16-token blocks the decode kernels serve the steps in which every
+// sequence schedules one token, and any other step goes to the generic kernel as a whole.
 bool decode_u8_shape(const pa_config& c) {
-    return c.kv_cache_dtype == PA_U8 && c.block_size == 32 && (c.head_size == 64 || c.head_size == 128) &&
-           c.num_heads / c.num_kv_heads <= 16;
+    return c.kv_cache_dtype == PA_U8 && (c.block_size == 32 || c.block_size == 16) &&
+           (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
@@ -277,7 +283,7 @@ bool mfma_shape(const pa_config& c) {
 
 // Shapes the 16-bit decode kernel is built for (single-token sequences of a call that asks for no scores).
 bool decode16_shape(const pa_config& c) {
-    return c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && c.block_size == 32 &&
+    return c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && (c.block_size == 32 || c.block_size == 16) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
@@ -299,8 +305,8 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
     auto plan = [&](int32_t waves, int32_t slots, int32_t* cap_out) {
         auto lds_of = [&](int32_t tiles) {
             int32_t off;
-            return u8 ? pa::decode_u8_lds_bytes(c.head_size, G, tiles, want_scores, waves, &off)
-                      : pa::decode16_lds_bytes(c.head_size, G, tiles, want_scores) + (size_t)tiles * sizeof(int32_t) + 16;
+            return u8 ? pa::decode_u8_lds_bytes(c.head_size, G, tiles, want_scores, waves, &off, c.block_size)
+                      : pa::decode16_lds_bytes(c.head_size, G, tiles, want_scores) + pa::decode16_table_bytes(tiles, c.block_size);
         };
         // the score path keeps a split's probabilities in LDS: that bounds the blocks per workgroup
         const size_t budget = (size_t)(160 * 1024 / (slots / 256)) - 1280;
@@ -330,7 +336,7 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
     // A context whose probabilities do not fit half a CU's LDS is cut into splits that send every head's
     // probabilities through HBM and add a merge.  With enough (sequence, kv head) pairs to give every CU a workgroup
     // of its own, one workgroup of eight waves per CU (the same waves per CU, the whole LDS) needs fewer of them.
-    if (u8 && most > cap4 && pairs >= 256) {
+    if (u8 && c.block_size == 32 && most > cap4 && pairs >= 256) {
         int32_t cap8 = 0;
         const int32_t s8 = plan(8, 256, &cap8);
         if (s8 < s) {
@@ -374,7 +380,9 @@ void plan_items(pa_ctx* ctx) {
     int32_t n_single_seqs = 0;
     std::vector<Tile> tiles;
     int64_t total_blocks = 0;
-    const bool split_off_decode = decode_u8_shape(ctx->cfg);
+    bool all_single = true;
+    for (int32_t b = 0; b < B; ++b) all_single = all_single && sb[b + 1] - sb[b] == 1;
+    const bool split_off_decode = decode_u8_shape(ctx->cfg) && (ctx->cfg.block_size == 32 || all_single);
     ctx->h_dec.clear();
     ctx->h_dec16.clear();
     for (int32_t b = 0; b < B; ++b) {
@@ -543,14 +551,16 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     // 16-bit caches, no dense chunk in the step: the single-token sequences go to their own decode kernel.  (Next to
     // dense chunks they stay work items of the matrix kernel: bandwidth-bound and matrix-bound items share the CUs
     // inside one launch, which two launches one after the other do not.)
-    const bool use_decode16 = use_mfma && decode16_shape(c) && !ctx->h_dec16.empty() &&
-                              ctx->n_single + ctx->n_sparse == ctx->n_items;
+    // (16-token blocks: the matrix kernel is out, the decode kernel serves the steps that are single-token throughout)
+    const bool use_decode16 = decode16_shape(c) && !ctx->h_dec16.empty() &&
+                              (c.block_size == 16 ? (int32_t)ctx->h_dec16.size() == ctx->B
+                                                  : use_mfma && ctx->n_single + ctx->n_sparse == ctx->n_items);
     const bool mfma_left = use_mfma && !(use_decode16 && ctx->n_single == ctx->n_items);
     if (static_ws)
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
                    PA_NOT_IMPLEMENTED,
                    "pa_attention_static serves steps in which every sequence schedules one token, over a u8 cache or a "
-                   "16-bit cache of the query's type (block size 32, head size 64 or 128, at most 16 heads per kv head)");
+                   "16-bit cache of the query's type (block size 32 or 16, head size 64 or 128, at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
     if (use_decode) {
@@ -680,7 +690,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
                                                decode_u8_shape(c) || use_decode16 ? 0 : 1, a.xatt));
     }
-    if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
+    if (use_decode || use_mfma || use_decode16) return;
     ctx->nsplit = ctx->generic_nsplit;
     ctx->part_acc.reserve(rows * ctx->nsplit * c.head_size * sizeof(float));
     ctx->part_ml.reserve(rows * ctx->nsplit * 2 * sizeof(float));

@@ -187,6 +187,58 @@ def test_decode16_kernel_shapes(pkg, dev, name, args, kw):
     assert np.array_equal(again["out16"], got["out16"])  # same kernel, same result, whatever ran in between
 
 
+BLOCK16 = [
+    # 16-token cache blocks: a 32-token tile of the decode kernels is two blocks (a last tile may hold one)
+    ("b16_u8_d128_g4", (8, 2, 128, 16, "f16", "u8", [0, 14, 15, 16, 17, 31, 32, 33, 47, 48, 49, 700], [1] * 12), {}),
+    ("b16_u8_d64_g8_bf16q", (16, 2, 64, 16, "bf16", "u8", [700, 64, 31, 16, 33, 1500], [1] * 6), {}),
+    ("b16_u8_multi_split", (8, 2, 128, 16, "f16", "u8", [3000, 2500, 17], [1, 1, 1]), {}),
+    ("b16_u8_window", (8, 2, 128, 16, "f16", "u8", [5000, 900, 40, 300], [1] * 4), {"sliding_window": 1000}),
+    ("b16_u8_window_unaligned", (8, 2, 128, 16, "f16", "u8", [300, 77, 23], [1] * 3), {"sliding_window": 45}),
+    ("b16_u8_g16_w0_mix", (16, 1, 128, 16, "f16", "u8", [300, 77, 500], [1] * 3), {"score_aggregation_window": [1, 0, 1]}),
+    ("b16_u8_long", (32, 8, 128, 16, "f16", "u8", [9000, 4100, 33], [1] * 3), {}),
+    ("b16_f16_d128_g4", (8, 2, 128, 16, "f16", "f16", [37, 130, 64, 4097, 0, 15, 16, 17, 31, 32, 33], [1] * 11), {}),
+    ("b16_bf16_d128_g7", (28, 4, 128, 16, "bf16", "bf16", [1000, 2047, 5], [1] * 3), {}),
+    ("b16_f16_d64_g1", (4, 4, 64, 16, "f16", "f16", [300, 64, 63, 1, 16], [1] * 5), {}),
+    ("b16_bf16_long_splits_window", (16, 8, 128, 16, "bf16", "bf16", [9000, 4000], [1, 1]), {"sliding_window": 2500}),
+    # a step with a multi-token sequence: no tuned kernel takes part of it, the generic one takes all of it
+    ("b16_u8_mixed_step", (8, 2, 128, 16, "f16", "u8", [300, 0, 77], [1, 40, 1]), {}),
+    ("b16_f16_mixed_step", (8, 2, 128, 16, "f16", "f16", [300, 0, 77], [1, 40, 1]), {}),
+]
+
+
+@pytest.mark.parametrize("name,args,kw", BLOCK16, ids=[c[0] for c in BLOCK16])
+def test_block_size_16_steps(pkg, dev, name, args, kw):
+    """Caches of 16-token blocks (the block size of the reference's GPU plugin): single-token steps on the decode
+    kernels, with and without scores, appended rows included; other steps on the generic kernel."""
+    got, ref, c = _check(pkg, dev, H.case_from_lens(name, *args, **kw), 59, outliers=True)
+    got2 = H.run_case_on_gpu(pkg, c, dev, want_scores=False)
+    H.assert_close(got2["out"], ref["out"], c["q_dtype"])
+    assert np.array_equal(got2["key_cache"], ref["key_cache"]) and np.array_equal(got2["value_cache"], ref["value_cache"])
+
+
+def test_block_size_16_runs_the_decode_kernels(pkg, dev):
+    """The tuned kernels, not the generic one, serve single-token steps over 16-token blocks: pa_attention_static, which
+    refuses every step the decode kernels do not take, accepts them and returns what pa_attention returns."""
+    import torch
+    for qd, kd in (("f16", "u8"), ("bf16", "bf16")):
+        c = H.build_case(H.case_from_lens(f"b16_which_{kd}", 8, 2, 128, 16, qd, kd, [5000, 3000, 15], [1, 1, 1]), 5)
+        op = pkg.PagedAttention(8, 2, 128, 16, qd, kd, 1, 0, torch.cuda.current_stream(dev))
+        q = H.to_device_16(torch, c["query"], qd, dev)
+        kc, vc = torch.from_numpy(c["key_cache0"]).to(dev), torch.from_numpy(c["value_cache0"]).to(dev)
+        op.step_begin(c["past_lens"], c["subsequence_begins"], c["block_indices_begins"],
+                      int((c["past_lens"] + c["new_lens"]).max()), c["score_aggregation_window"], 0, c["scale"])
+        op.set_block_indices(c["block_indices"], c["num_blocks"])
+        outs = []
+        for call in (op.attention_static, op.attention):
+            out = torch.full_like(q, float("nan"))
+            scores = torch.full((op.total_scores,), float("nan"), dtype=torch.float32, device=dev)
+            call(q, kc, vc, out, scores)
+            op.synchronize()
+            outs.append((out.view(torch.int16).cpu().numpy(), scores.cpu().numpy()))
+        assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+        assert np.isfinite(outs[0][1]).all()
+
+
 _SHORT = list(range(5, 1500, 23))
 WIDE_WORKGROUP = [
     # (name, args, kw, splits): contexts whose probabilities do not fit half a CU's LDS, in steps with at least 256

@@ -68,12 +68,19 @@ __device__ __forceinline__ void swap_rows16(float& a, float& b) {
 __device__ __forceinline__ void swap_halves32(float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
+// (the maxima as instructions of their own: behind the lane swaps the compiler no longer knows its operands to be
+// ordinary numbers and puts a quieting `v_max x, x, x` in front of every fmaxf)
+__device__ __forceinline__ float max_raw(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 __device__ __forceinline__ float xor_max_g(float v) {
     float a = v, b = v;
     swap_rows16(a, b);
-    a = b = fmaxf(a, b);
+    a = b = max_raw(a, b);
     swap_halves32(a, b);
-    return fmaxf(a, b);
+    return max_raw(a, b);
 }
 __device__ __forceinline__ float xor_sum_g(float v) {
     float a = v, b = v;
@@ -521,7 +528,8 @@ void pa_prefill16_kernel(PrefillArgs a) {
 #pragma unroll
             for (int jj = 0; jj < (U8 ? 0 : 4); ++jj) {
                 // second operand: what the rounding to the operand type dropped
-                const uint32_t hi = pack2<DT>(p[2 * jj], p[2 * jj + 1]);
+                uint32_t hi = pack2<DT>(p[2 * jj], p[2 * jj + 1]);
+                if (DT == DT_BF16) asm("" : "+v"(hi));  // (its halves are taken from this word, not converted once more)
                 pb[gi][jj] = hi;
                 if (DT == DT_BF16) {
                     pl[gi][jj] = pack2<DT>(p[2 * jj] - __builtin_bit_cast(float, hi << 16),
@@ -628,8 +636,12 @@ void pa_prefill16_kernel(PrefillArgs a) {
         const int my_piece2 = ((lane & 15) ^ ((my_row + 4) & 15)) << 4;
         const int my_vpiece = ((lane & 15) ^ ((my_row & 7) << 1)) << 4;
         const int my_vpiece2 = ((lane & 15) ^ (((my_row + 4) & 7) << 1)) << 4;
+        // (the block id of a copy is read one step before the copy goes out: a scalar load that is waited for right behind
+        // its issue stalls the wave at the start of every step)
+        int id_next = 0;
         auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
-            const long blk = ((long)table[tile_at(j)] * Hkv + hkv) * (TOK * CROWB);
+            const long blk = ((long)id_next * Hkv + hkv) * (TOK * CROWB);
+            id_next = table[tile_at(j + 1)];
             const uint8_t* kg = a.key_cache + blk + my_row * ROWB;
             const uint8_t* vg = a.value_cache + blk + my_row * ROWB;
             uint8_t* kd = kslot_base + wv * 2048;
@@ -639,6 +651,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
             dma16(vg + my_vpiece, vd);
             dma16(vg + 4 * ROWB + my_vpiece2, vd + 1024);
         };
+        id_next = table[tile_at(0)];
         copy_in(0, dk0, dv0);
         copy_in(1, dk1, dv1);
         copy_in(2, dk2, dv2);

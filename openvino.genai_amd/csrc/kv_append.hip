@@ -1,8 +1,8 @@
 // KV append: writes the new tokens' K and V rows into the block-tabled caches.
 //
-// One 64-lane wave owns one (token, kv head, K|V) row of D elements, so the row's min/max is a
-// wave reduction and the row is written as one contiguous, coalesced burst.  HBM-bound byte work:
-// each input element is read once and each cache byte written once.
+// Sixteen lanes own one (token, kv head, K|V) row of D elements, so the row's min/max is a reduction over 16 lanes
+// and a wave writes four rows.  HBM-bound byte work: each input element is read once and each cache byte written
+// once.
 //
 // u8 rows are `f32 scale | f32 zero-point | D codes` with
 //   scale = (max - min) / 255  (a zero range takes 1e-4),  zp = -min / scale,
@@ -13,40 +13,102 @@
 namespace pa {
 namespace {
 
-template <int QDT, int KVDT, int EPL>
+// A row per 16 lanes, each lane D / 16 consecutive elements (16-byte loads at D = 128), four rows per wave.  A wave
+// takes four consecutive tokens of one kv head, so that what it writes is one run of cache bytes wherever the
+// tokens share a block.  Minimum and maximum of a row are reduced over its 16 lanes with four
+// cross-lane (DPP) steps; the arithmetic per element is that of quantize_row_u8, so the bytes are the same.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_min(float v) {
+    v = fminf(v, dpp_f<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+    v = fminf(v, dpp_f<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+    v = fminf(v, dpp_f<0x141>(v));  // row_half_mirror: the other quad of the eight
+    return fminf(v, dpp_f<0x140>(v));  // row_mirror: the other eight of the sixteen
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    v = fmaxf(v, dpp_f<0x141>(v));
+    return fmaxf(v, dpp_f<0x140>(v));
+}
+
+template <int QDT, int KVDT, int E>
 __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ key,
                                                         const uint16_t* __restrict__ value,
                                                         uint8_t* __restrict__ key_cache,
                                                         uint8_t* __restrict__ value_cache,
                                                         const int32_t* __restrict__ block_indices) {
-    const int lane = threadIdx.x & 63;
-    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const long rows = (long)st.T * sh.Hkv * 2;
-    if (row >= rows) return;
-    const int which = (int)(row & 1);
-    const int h = (int)((row >> 1) % sh.Hkv);
-    const int t = (int)((row >> 1) / sh.Hkv);
+#pragma clang fp contract(off)
+    static_assert(E == 4 || E == 8, "D = 64 or 128");
+    constexpr int D = 16 * E;
+    const int l16 = threadIdx.x & 15;
+    const long per_tensor = (long)st.T * sh.Hkv;
+    long row = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;  // (K | V, kv head, token)
+    // (rows beyond the end repeat the last one: no divergence around the cross-lane steps, and the same bytes twice)
+    row = min(row, 2 * per_tensor - 1);
+    const int which = row >= per_tensor;
+    const long rem = row - which * per_tensor;
+    const int h = (int)(rem / st.T), t = (int)(rem % st.T);
     const int b = st.token_seq[t];
     const int slot = st.past_lens[b] + (t - st.subsequence_begins[b]);
     const long phys = block_indices[st.block_indices_begins[b] + slot / sh.bs];
-    const int D = sh.D;
-    const int rb = row_bytes(D, KVDT);
-    const uint16_t* src = (which ? value : key) + ((long)t * sh.Hkv + h) * D + lane * EPL;
-    uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)rb;
+    constexpr int RB = KVDT == DT_U8 ? D + 8 : 2 * D;
+    const uint16_t* src = (which ? value : key) + ((long)t * sh.Hkv + h) * D + l16 * E;
+    uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)RB;
 
-    uint16_t raw[EPL];
-    load_row16<EPL>(src, raw);
-
-    if (KVDT == DT_U8) {
-        quantize_row_u8<QDT, EPL>(raw, dst, lane);
+    uint32_t w[E / 2];
+    if constexpr (E == 4) {
+        const uint2 v = *reinterpret_cast<const uint2*>(src);
+        w[0] = v.x; w[1] = v.y;
     } else {
-        uint16_t o[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) o[e] = (QDT == KVDT) ? raw[e] : store16<KVDT>(load16<QDT>(raw[e]));
-        uint16_t* c = reinterpret_cast<uint16_t*>(dst) + lane * EPL;
-        if constexpr (EPL == 4) *reinterpret_cast<uint2*>(c) = make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
-        else if constexpr (EPL == 2) *reinterpret_cast<uint32_t*>(c) = o[0] | ((uint32_t)o[1] << 16);
-        else *c = o[0];
+        for (int i = 0; i < E / 8; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(src + 8 * i);
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+        }
+    }
+    if constexpr (KVDT == DT_U8) {
+        float x[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[e] = load16<QDT>((uint16_t)(w[e / 2] >> (16 * (e & 1))));
+        float mn = x[0], mx = x[0];
+#pragma unroll
+        for (int e = 1; e < E; ++e) { mn = fminf(mn, x[e]); mx = fmaxf(mx, x[e]); }
+        mn = row16_min(mn);
+        mx = row16_max(mx);
+        float scale = (mx - mn) / 255.0f;
+        if (scale == 0.0f) scale = 0.0001f;
+        const float zp = -mn / scale;
+        const float inv = 1.0f / scale;
+        uint32_t codes[E / 4];
+#pragma unroll
+        for (int i = 0; i < E / 4; ++i) codes[i] = 0;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float v = rintf(__fmaf_rn(x[e], inv, zp));
+            v = fminf(fmaxf(v, 0.0f), 255.0f);
+            codes[e / 4] |= (uint32_t)(int)v << (8 * (e & 3));
+        }
+        if (l16 == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
+        uint8_t* c = dst + 8 + l16 * E;  // rows are multiples of 8 bytes
+        if constexpr (E == 4) *reinterpret_cast<uint32_t*>(c) = codes[0];
+        else
+#pragma unroll
+            for (int i = 0; i < E / 8; ++i) *reinterpret_cast<uint2*>(c + 8 * i) = make_uint2(codes[2 * i], codes[2 * i + 1]);
+    } else {
+        if constexpr (QDT != KVDT) {
+#pragma unroll
+            for (int i = 0; i < E / 2; ++i)
+                w[i] = (uint32_t)store16<KVDT>(load16<QDT>((uint16_t)(w[i] & 0xffff))) |
+                       ((uint32_t)store16<KVDT>(load16<QDT>((uint16_t)(w[i] >> 16))) << 16);
+        }
+        uint8_t* c = dst + l16 * E * 2;
+        if constexpr (E == 4) *reinterpret_cast<uint2*>(c) = make_uint2(w[0], w[1]);
+        else
+#pragma unroll
+            for (int i = 0; i < E / 8; ++i) *reinterpret_cast<uint4*>(c + 16 * i) = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
     }
 }
 
@@ -55,15 +117,14 @@ hipError_t launch_epl(hipStream_t s, const StepDev& st, const Shape& sh, const v
                       void* kc, void* vc, const int32_t* bi) {
     const long rows = (long)st.T * sh.Hkv * 2;
     if (rows == 0) return hipSuccess;
-    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    dim3 grid((unsigned)((rows + 15) / 16)), block(256);
     auto k = reinterpret_cast<const uint16_t*>(key);
     auto v = reinterpret_cast<const uint16_t*>(value);
     auto kcu = reinterpret_cast<uint8_t*>(kc);
     auto vcu = reinterpret_cast<uint8_t*>(vc);
     switch (sh.D / 64) {
-        case 1: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 1>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
-        case 2: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 2>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
-        case 4: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 4>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        case 1: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 4>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        case 2: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 8>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

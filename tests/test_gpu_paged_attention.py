@@ -42,6 +42,48 @@ def test_kv_append_bit_exact(pkg, dev, qd, kd, D):
     _check(pkg, dev, case, 3, outliers=True, want_scores=False)
 
 
+MANY_ROWS = [
+    # (query type, cache type, D, Hkv, block size): steps of 16384 or more (token, kv head, K | V) rows take the
+    # append kernel with a row per 16 lanes
+    ("f16", "u8", 128, 4, 32), ("bf16", "u8", 128, 8, 32), ("f16", "u8", 64, 4, 32), ("bf16", "u8", 64, 2, 32),
+    ("f16", "u8", 128, 4, 16), ("f16", "f16", 128, 4, 32), ("bf16", "bf16", 64, 4, 32), ("f16", "bf16", 128, 4, 32),
+    ("bf16", "f16", 64, 2, 16),
+]
+
+
+@pytest.mark.parametrize("qd,kd,D,Hkv,bs", MANY_ROWS)
+def test_kv_append_many_rows_bit_exact(pkg, dev, qd, kd, D, Hkv, bs):
+    import torch
+    from oracle import oracle as O
+    T_min = 16384 // (2 * Hkv) + 70
+    new = [T_min - 700, 333, 1, 300, 65, 1]
+    case = H.case_from_lens(f"append_many_{qd}_{kd}_{D}", Hkv, Hkv, D, bs, qd, kd, [0, 31, 4000, 100, 7, 0], new)
+    print(f"case {case['name']} seed 9", flush=True)
+    c = H.build_case(case, 9, outliers=True)
+    assert int(c["subsequence_begins"][-1]) * Hkv * 2 >= 16384
+    # rows with a zero range, a huge range and exact ties, in the middle of the long sequence
+    x = np.zeros((3, Hkv * D), np.float32)
+    x[0] = 3.25
+    x[1, ::2], x[1, 1::2] = -60000.0, 60000.0
+    x[2] = np.tile(np.arange(D, dtype=np.float32) * 0.5, Hkv)
+    c["key"][500:503] = O.to_bits(x, H.DT[qd])
+    c["value"][800:803] = O.to_bits(x[::-1].copy(), H.DT[qd])
+    kc_ref, vc_ref = c["key_cache0"].copy(), c["value_cache0"].copy()
+    O.kv_append(c["key"], c["value"], H.DT[qd], kc_ref, vc_ref, H.DT[kd], c["past_lens"], c["subsequence_begins"],
+                c["block_indices"], c["block_indices_begins"], Hkv, D, bs)
+    op = pkg.PagedAttention(Hkv, Hkv, D, bs, qd, kd, 1, 0, torch.cuda.current_stream(dev))
+    k = H.to_device_16(torch, c["key"], qd, dev)
+    v = H.to_device_16(torch, c["value"], qd, dev)
+    kc, vc = torch.from_numpy(c["key_cache0"]).to(dev), torch.from_numpy(c["value_cache0"]).to(dev)
+    op.step_begin(c["past_lens"], c["subsequence_begins"], c["block_indices_begins"],
+                  int((c["past_lens"] + c["new_lens"]).max()))
+    op.set_block_indices(c["block_indices"], c["num_blocks"])
+    op.kv_append(k, v, kc, vc)
+    op.synchronize()
+    assert np.array_equal(kc.cpu().numpy(), kc_ref), "key cache bytes differ"
+    assert np.array_equal(vc.cpu().numpy(), vc_ref), "value cache bytes differ"
+
+
 def test_kv_append_constant_and_extreme_rows(pkg, dev):
     # constant rows (zero range), huge range, and exact .5 ties
     import torch

@@ -265,10 +265,8 @@ void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
                                    ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
 }
 
-// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).  Its tiles are 32
-// tokens: one 32-token cache block or two 16-token ones.  The matrix kernel that takes the other sequences of a step
-// is built for 32-token blocks only, so with 16-token blocks the decode kernels serve the steps in which every
-// sequence schedules one token, and any other step goes to the generic kernel as a whole.
+// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).  The tuned kernels'
+// tiles are 32 tokens: one 32-token cache block or two 16-token ones.
 bool decode_u8_shape(const pa_config& c) {
     return c.kv_cache_dtype == PA_U8 && (c.block_size == 32 || c.block_size == 16) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
@@ -277,7 +275,7 @@ bool decode_u8_shape(const pa_config& c) {
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
 bool mfma_shape(const pa_config& c) {
-    return (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && c.block_size == 32 &&
+    return (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && (c.block_size == 32 || c.block_size == 16) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 256;
 }
 
@@ -380,9 +378,7 @@ void plan_items(pa_ctx* ctx) {
     int32_t n_single_seqs = 0;
     std::vector<Tile> tiles;
     int64_t total_blocks = 0;
-    bool all_single = true;
-    for (int32_t b = 0; b < B; ++b) all_single = all_single && sb[b + 1] - sb[b] == 1;
-    const bool split_off_decode = decode_u8_shape(ctx->cfg) && (ctx->cfg.block_size == 32 || all_single);
+    const bool split_off_decode = decode_u8_shape(ctx->cfg);
     ctx->h_dec.clear();
     ctx->h_dec16.clear();
     for (int32_t b = 0; b < B; ++b) {
@@ -551,10 +547,8 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     // 16-bit caches, no dense chunk in the step: the single-token sequences go to their own decode kernel.  (Next to
     // dense chunks they stay work items of the matrix kernel: bandwidth-bound and matrix-bound items share the CUs
     // inside one launch, which two launches one after the other do not.)
-    // (16-token blocks: the matrix kernel is out, the decode kernel serves the steps that are single-token throughout)
-    const bool use_decode16 = decode16_shape(c) && !ctx->h_dec16.empty() &&
-                              (c.block_size == 16 ? (int32_t)ctx->h_dec16.size() == ctx->B
-                                                  : use_mfma && ctx->n_single + ctx->n_sparse == ctx->n_items);
+    const bool use_decode16 = use_mfma && decode16_shape(c) && !ctx->h_dec16.empty() &&
+                              ctx->n_single + ctx->n_sparse == ctx->n_items;
     const bool mfma_left = use_mfma && !(use_decode16 && ctx->n_single == ctx->n_items);
     if (static_ws)
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
@@ -690,7 +684,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
                                                decode_u8_shape(c) || use_decode16 ? 0 : 1, a.xatt));
     }
-    if (use_decode || use_mfma || use_decode16) return;
+    if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;
     ctx->part_acc.reserve(rows * ctx->nsplit * c.head_size * sizeof(float));
     ctx->part_ml.reserve(rows * ctx->nsplit * 2 * sizeof(float));
@@ -941,7 +935,7 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
             if (had) plan_items(ctx);
             return;
         }
-        PA_REQUIRE(mfma_shape(c), PA_NOT_IMPLEMENTED,
+        PA_REQUIRE(mfma_shape(c) && c.block_size == 32, PA_NOT_IMPLEMENTED,
                    "block-sparse prefill needs block_size 32, head_size 64 or 128 and a u8 cache or one of the query's type");
         auto pow2 = [](int32_t v) { return v > 0 && (v & (v - 1)) == 0; };
         PA_REQUIRE(pow2(block_size) && block_size >= 32, PA_NOT_IMPLEMENTED,

@@ -324,8 +324,20 @@ void pa_prefill16_kernel(PrefillArgs a) {
     const int ltid = tid % NCH;
     const int lds_k = (ltid / CPR) * LROWK + (ltid % CPR) * 16;
     const int lds_v = OFF_V + (ltid / CPR) * LROWV + (ltid % CPR) * 16;
+    const int kv_len = past + st.subsequence_begins[b + 1] - t0;
+    // The kernel's tiles are 32 tokens: one 32-token cache block, or two 16-token blocks, in which case each row is
+    // fetched from the block it lies in (a last tile of one block repeats it; those rows lie beyond kv_len).
+    // tile_base(tile, upper): what to add to `row * CROWB` for a row of the tile's lower or upper half.
+    const bool bs16 = a.sh.bs == 16;
+    const int last_block16 = (kv_len - 1) >> 4;
+    auto tile_base = [&](int tile, bool upper) __attribute__((always_inline)) -> long {
+        if (!bs16) return ((long)table[tile] * Hkv + hkv) * (TOK * CROWB);
+        const long lo = ((long)table[2 * tile] * Hkv + hkv) * (16 * CROWB);
+        const long hi = ((long)table[min(2 * tile + 1, last_block16)] * Hkv + hkv) * (16 * CROWB) - 16 * CROWB;
+        return upper ? hi : lo;
+    };
     auto fetch = [&](KvRegs<U8>& r, int j) __attribute__((always_inline)) {
-        const long blk = ((long)table[tile_at(j)] * Hkv + hkv) * (TOK * CROWB);
+        const long blk = tile_base(tile_at(j), ltid / CPR >= 16);
         if constexpr (U8) {
             const long row = blk + (long)(ltid / CPR) * CROWB;
             kv_issue(r, a.key_cache + row, a.value_cache + row, 8 + (ltid % CPR) * 8);
@@ -333,7 +345,6 @@ void pa_prefill16_kernel(PrefillArgs a) {
             kv_issue(r, a.key_cache + blk + (long)ltid * 16, a.value_cache + blk + (long)ltid * 16);
         }
     };
-    const int kv_len = past + st.subsequence_begins[b + 1] - t0;
     // rows beyond the sequence's tokens (the tail of its last block) may hold anything: their K columns are masked
     // by the causal select, their V rows are cleared here so that 0 * garbage cannot reach the accumulators
     // j = block number within the item's range; it selects the LDS slots
@@ -638,10 +649,11 @@ void pa_prefill16_kernel(PrefillArgs a) {
         const int my_vpiece2 = ((lane & 15) ^ (((my_row + 4) & 7) << 1)) << 4;
         // (the block id of a copy is read one step before the copy goes out: a scalar load that is waited for right behind
         // its issue stalls the wave at the start of every step)
-        int id_next = 0;
+        const bool upper_half = __builtin_amdgcn_readfirstlane(wv) >= (NT / 64) / 2;  // this wave moves rows 16 - 31
+        long base_next = 0;
         auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
-            const long blk = ((long)id_next * Hkv + hkv) * (TOK * CROWB);
-            id_next = table[tile_at(j + 1)];
+            const long blk = base_next;
+            base_next = tile_base(tile_at(j + 1), upper_half);
             const uint8_t* kg = a.key_cache + blk + my_row * ROWB;
             const uint8_t* vg = a.value_cache + blk + my_row * ROWB;
             uint8_t* kd = kslot_base + wv * 2048;
@@ -651,7 +663,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
             dma16(vg + my_vpiece, vd);
             dma16(vg + 4 * ROWB + my_vpiece2, vd + 1024);
         };
-        id_next = table[tile_at(0)];
+        base_next = tile_base(tile_at(0), upper_half);
         copy_in(0, dk0, dv0);
         copy_in(1, dk1, dv1);
         copy_in(2, dk2, dv2);

@@ -74,6 +74,7 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
     if (base >= kv_len) return;
     const int W = st.score_window[b];
     const int Hq = sh.Hq, Hkv = sh.Hkv, G = Hq / Hkv;
+    const int bs_shift = sh.bs == 16 ? 4 : 5;  // cache blocks of 16 or 32 tokens
     const int R = W * G;                       // query rows per kv head
     const int first_tok = t0 + q_len - W;      // first of the last W tokens
     const int first_pos = past + q_len - W;    // its position
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
                 // out back to back (behind a branch each load was waited for before the next was issued); such
                 // columns are masked below, where every row's limit is below kv_len
                 const int pos = min(base + 16 * c + n, kv_len - 1);
-                const uint8_t* row = key_cache + (((long)table[pos >> 5] * Hkv + hkv) * 32 + (pos & 31)) * CROWB;
+                const uint8_t* row = key_cache + (((long)table[pos >> bs_shift] * Hkv + hkv) * sh.bs + (pos & (sh.bs - 1))) * CROWB;
                 if (U8) {
                     const float2 hd = *reinterpret_cast<const float2*>(row);
                     sck[c] = hd.x * scl * CODE_UNIT;
@@ -210,7 +211,7 @@ hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& s
                            block_indices, final_ml, scores, single_token_too, xd);                             \
         return hipGetLastError();                                                                              \
     }
-    if (sh.bs != 32) return hipErrorInvalidValue;
+    if (sh.bs != 32 && sh.bs != 16) return hipErrorInvalidValue;
     if (kv_dtype == DT_U8) {
         if (sh.D == 64 && q_dtype == DT_F16) PA_REPLAY(64, DT_F16, DT_F16, true)
         if (sh.D == 64 && q_dtype == DT_BF16) PA_REPLAY(64, DT_F16, DT_BF16, true)

@@ -21,7 +21,8 @@ def big_case(rng, idx):
             new.append(int(rng.integers(2, 700)))
     sw = int(rng.choice([0, 0, 0, int(rng.integers(64, 5000))]))
     saw = [int(rng.integers(0, min(n, 16) + 1)) for n in new] if rng.random() < 0.7 else None
-    return H.case_from_lens(f"big_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_sw{sw}", Hkv * G, Hkv, D, 32, qd, kd, past, new,
+    bs = 16 if idx % 4 == 3 else 32  # (from the index, not the generator: the other cases stay what they were)
+    return H.case_from_lens(f"big_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_sw{sw}_b{bs}", Hkv * G, Hkv, D, bs, qd, kd, past, new,
                             sliding_window=sw, score_aggregation_window=saw)
 
 
@@ -39,7 +40,8 @@ def peaked_case(rng, idx):
             past.append(int(rng.choice([0, int(rng.integers(1, 5000))])))
             new.append(int(rng.integers(2, 300)))
     mult = float(rng.choice([2.0, 4.0, 8.0]))
-    return H.case_from_lens(f"peaked_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_x{mult}", Hkv * G, Hkv, D, 32, qd, kd, past, new,
+    bs = 16 if idx % 4 == 3 else 32
+    return H.case_from_lens(f"peaked_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_x{mult}_b{bs}", Hkv * G, Hkv, D, bs, qd, kd, past, new,
                             scale=mult / np.sqrt(D))
 
 

@@ -242,16 +242,27 @@ BLOCK16 = [
     ("b16_bf16_d128_g7", (28, 4, 128, 16, "bf16", "bf16", [1000, 2047, 5], [1] * 3), {}),
     ("b16_f16_d64_g1", (4, 4, 64, 16, "f16", "f16", [300, 64, 63, 1, 16], [1] * 5), {}),
     ("b16_bf16_long_splits_window", (16, 8, 128, 16, "bf16", "bf16", [9000, 4000], [1, 1]), {"sliding_window": 2500}),
-    # a step with a multi-token sequence: no tuned kernel takes part of it, the generic one takes all of it
+    # steps with multi-token sequences: the matrix kernel's 32-token tiles are two blocks as well
     ("b16_u8_mixed_step", (8, 2, 128, 16, "f16", "u8", [300, 0, 77], [1, 40, 1]), {}),
     ("b16_f16_mixed_step", (8, 2, 128, 16, "f16", "f16", [300, 0, 77], [1, 40, 1]), {}),
+    ("b16_bf16_g7_mixed", (28, 4, 128, 16, "bf16", "bf16", [0, 700, 333, 40, 2000], [150, 37, 1, 1, 64]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3]}),
+    ("b16_f16_d64_g8", (32, 4, 64, 16, "f16", "f16", [0, 15, 16, 500], [33, 100, 1, 17]), {}),
+    ("b16_f16_chunks_only_window", (4, 4, 128, 16, "f16", "f16", [300, 0], [200, 130]), {"sliding_window": 100}),
+    ("b16_bf16_long_chunk", (6, 2, 128, 16, "bf16", "bf16", [1500], [700]), {"score_aggregation_window": [16]}),
+    ("b16_u8_g4_mixed", (32, 8, 128, 16, "f16", "u8", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
+    ("b16_u8_bf16q_d64_g8", (16, 2, 64, 16, "bf16", "u8", [0, 31, 16, 500], [33, 100, 1, 17]), {}),
+    ("b16_u8_window", (8, 2, 128, 16, "f16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
+    ("b16_u8_odd_block_counts", (8, 2, 128, 16, "f16", "u8", [0, 3, 20], [17, 45, 60]), {}),
 ]
 
 
 @pytest.mark.parametrize("name,args,kw", BLOCK16, ids=[c[0] for c in BLOCK16])
 def test_block_size_16_steps(pkg, dev, name, args, kw):
-    """Caches of 16-token blocks (the block size of the reference's GPU plugin): single-token steps on the decode
-    kernels, with and without scores, appended rows included; other steps on the generic kernel."""
+    """Caches of 16-token blocks (the block size of the reference's GPU plugin) on the tuned kernels, whose 32-token
+    tiles are then two blocks: single-token steps, chunks and mixed steps, with and without scores, appended rows
+    included."""
     got, ref, c = _check(pkg, dev, H.case_from_lens(name, *args, **kw), 59, outliers=True)
     got2 = H.run_case_on_gpu(pkg, c, dev, want_scores=False)
     H.assert_close(got2["out"], ref["out"], c["q_dtype"])

@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--config", type=int, default=2, help="workload (2 = headline; 1, 4, 5 for diagnostics)")
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--sliding-window", type=int, default=None)
+    ap.add_argument("--block-size", type=int, choices=[16, 32], default=None,
+                    help="KV block size of the workload (default: the configuration's, 32)")
     ap.add_argument("--kv-dtype", choices=["u8", "f16", "bf16"], default=None,
                     help="diagnostics: run the workload's shape over another cache type")
     ap.add_argument("--no-scores", action="store_true")
@@ -368,7 +370,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    spec = wl.make_spec(args.config, batch=args.batch, sliding_window=args.sliding_window, pool_factor=args.pool_factor)
+    spec = wl.make_spec(args.config, batch=args.batch, sliding_window=args.sliding_window, pool_factor=args.pool_factor,
+                        block_size=args.block_size)
+    if args.block_size is not None and args.block_size != 32:
+        spec["name"] += "_block%d" % args.block_size
     if args.pool_factor != 2.0:
         spec["name"] += "_pool%g" % args.pool_factor
     if args.kv_dtype and args.kv_dtype != spec["kv_dtype"]:

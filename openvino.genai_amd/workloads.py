@@ -25,7 +25,7 @@ CONFIGS = {
 }
 
 
-def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0):
+def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0, block_size=None):
     """Step metadata of config ``cfg`` (1..5); ``batch`` / ``context_scale`` shrink it for parity tests."""
     c = dict(CONFIGS[cfg])
     rng = np.random.Generator(np.random.PCG64(1000 + cfg if seed is None else seed))
@@ -45,7 +45,7 @@ def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None
         past = np.concatenate([[sc(p) for p in chunk_pasts], rng.integers(sc(lo), sc(hi) + 1, size=n_dec)])
         new = np.concatenate([np.full(len(chunk_pasts), max(1, sc(chunk_len))), np.ones(n_dec, np.int64)])
         B = len(past)
-    bs = c["bs"]
+    bs = c["bs"] if block_size is None else int(block_size)
     nblk = (past + new + bs - 1) // bs
     bib = np.concatenate([[0], np.cumsum(nblk)])
     pool = int(np.ceil(pool_factor * bib[-1]))

@@ -275,7 +275,23 @@ struct PrefillArgs {
     int32_t n_single;
     const int32_t* single_idx;    // [B]: index among the single-token sequences, -1 for the others
     int32_t skip_single;
+    // Scores of single-token sequences that are work items of this kernel (16-bit caches, next to dense chunks): the
+    // kernel keeps every head's probabilities, relative to the running maximum at their 32-token tile, and that
+    // maximum per (head, tile) in LDS while it walks an item, and leaves them here when the item is done;
+    // `launch_single_scores` turns them into scores once the rows' final maxima and denominators are known.  Null:
+    // nothing is left (the score replay serves those sequences).
+    _Float16* p_out;              // [tiles][Hq][32]: a sequence's tiles start at tile_max_offset(score offset, b)
+    float* tile_max;              // [tiles][Hq]
 };
+// What an item of a single-token sequence may keep in LDS: 64 G bytes of probabilities and 4 G of maxima per tile.
+constexpr int SINGLE_STASH_BYTES = 20480;
+__host__ __device__ inline int single_item_max_tiles(int G) { return SINGLE_STASH_BYTES / (68 * G); }
+// Tiles of the sequences of a step, one after the other: a sequence of kv_len positions takes ceil(kv_len / 32).
+__host__ __device__ inline long tile_max_offset(long score_offset, int b) { return (score_offset >> 5) + b; }
+__host__ __device__ inline long tile_max_count(long total_scores, int B) { return (total_scores >> 5) + B + 1; }
+// Scores of the listed single-token sequences from what the matrix kernel left (after its merge kernel).
+hipError_t launch_single_scores(hipStream_t s, const PrefillArgs& a, const int32_t* seq_list, int n_seqs, float* scores,
+                                int max_kv_len);
 hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, int kv_dtype, hipEvent_t ev0,
                             hipEvent_t ev1);
 

@@ -127,6 +127,8 @@ struct pa_ctx {
     std::vector<int32_t> h_dec;
     std::vector<int32_t> h_dec16;     // single-token sequences of a 16-bit-cache step (also listed as matrix-kernel items)
     DevBuf dec16_list;
+    DevBuf tile_max;   // per (head, 32-token tile) maxima of single-token sequences handled by the matrix kernel
+    bool stash_ok = false;  // the step's single-token items are short enough to keep their probabilities in LDS
     int32_t n_items = 0, n_wide = 0, max_split = 1;
     size_t tok_nsplit_off = 0;
     // single-token sequences the matrix kernel may take (16-bit caches): their work items, and behind the split
@@ -400,6 +402,9 @@ void plan_items(pa_ctx* ctx) {
         }
     }
     const int64_t target = std::min<int64_t>(128, std::max<int64_t>(8, total_blocks * ctx->cfg.num_kv_heads / 768));
+    // single-token sequences as items of the kernel variant that can hand their probabilities to the score kernel
+    const bool stash_ok = narrow_all && G <= 16;
+    ctx->stash_ok = stash_ok;
     std::vector<pa::PrefillItem>& items = ctx->h_items;
     items.clear();
     std::vector<int32_t> tok_ns(T, 1);
@@ -410,7 +415,9 @@ void plan_items(pa_ctx* ctx) {
     ctx->n_single = 0;
     for (const Tile& t : tiles) {
         const int32_t nt = t.hi - t.lo;
-        const int32_t per = (int32_t)((nt + (nt + target - 1) / target - 1) / ((nt + target - 1) / target));
+        // (items of single-token sequences over 16-bit caches keep their probabilities in LDS when scores are wanted)
+        const int64_t most = t.kind == 2 && stash_ok ? std::min<int64_t>(target, pa::single_item_max_tiles(G)) : target;
+        const int32_t per = (int32_t)((nt + (nt + most - 1) / most - 1) / ((nt + most - 1) / most));
         const int32_t ns = (nt + per - 1) / per;
         for (int32_t s = 0; s < ns; ++s)
             items.push_back({t.b, t.q0, t.nq, t.lo + s * per, std::min(t.hi, t.lo + (s + 1) * per), s, ns, 0});
@@ -675,14 +682,29 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
             HIP_CHECK(pa::launch_xattention(ctx->stream, x, c.query_dtype, c.kv_cache_dtype));
             ctx->x_ran = true;
         }
+        // Single-token sequences that are work items of this launch (16-bit caches, next to dense chunks): with scores
+        // wanted the kernel leaves their probabilities for a small score kernel, instead of a replay that reads all
+        // their K rows once more.
+        const bool hand_over = io->scores && ctx->stash_ok && !use_decode16 && ctx->n_single > 0;
+        if (hand_over) {
+            const size_t tiles = (size_t)pa::tile_max_count(ctx->total_scores, ctx->B);
+            ctx->p_split.reserve(tiles * c.num_heads * 32 * sizeof(uint16_t));
+            ctx->tile_max.reserve(tiles * c.num_heads * sizeof(float));
+            a.p_out = ctx->p_split.as<_Float16>();
+            a.tile_max = ctx->tile_max.as<float>();
+        }
         if (!use_decode && !use_decode16) ctx->nsplit = ctx->max_split;
         HIP_CHECK(pa::launch_prefill16(ctx->stream, a, c.query_dtype, c.kv_cache_dtype, ev0, ev1));
         ctx->timed = ctx->profiling;
-        // scores of the multi-token sequences (and of single-token ones that were work items of this kernel): replay
+        if (hand_over)
+            HIP_CHECK(pa::launch_single_scores(ctx->stream, a, ctx->dec16_list.as<int32_t>(), (int)ctx->h_dec16.size(),
+                                               io->scores, ctx->max_kv));
+        // scores of the multi-token sequences (and of single-token ones that were work items of this kernel and left
+        // nothing for the score kernel): replay
         if (io->scores && !(use_decode16 && ctx->n_single == ctx->n_items))
             HIP_CHECK(pa::launch_scores_replay(ctx->stream, ctx->dev, a.sh, c.query_dtype, c.kv_cache_dtype, io->query,
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
-                                               decode_u8_shape(c) || use_decode16 ? 0 : 1, a.xatt));
+                                               decode_u8_shape(c) || use_decode16 || hand_over ? 0 : 1, a.xatt));
     }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;
@@ -738,6 +760,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->pf_part_ml.release();
     ctx->dec_list.release();
     ctx->dec16_list.release();
+    ctx->tile_max.release();
     ctx->trig_lut.release();
     ctx->rot_args.release();
     ctx->div_seqs.release();

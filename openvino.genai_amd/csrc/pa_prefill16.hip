@@ -202,7 +202,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
     __shared__ __align__(16) uint8_t dk0[DMA ? TILEK : 16], dk1[DMA ? TILEK : 16], dk2[DMA ? TILEK : 16], dk3[DMA ? TILEK : 16];
     __shared__ __align__(16) uint8_t dv0[DMA ? TILEV : 16], dv1[DMA ? TILEV : 16], dv2[DMA ? TILEV : 16], dv3[DMA ? TILEV : 16];
     auto kslot = [](int j) { return (j & 1); };
-    auto vslot = [](int j) { return (j & 3); };
+    auto vslot = [](int j) { return (j & (NVS - 1)); };
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -395,6 +395,14 @@ void pa_prefill16_kernel(PrefillArgs a) {
         }
     };
     const bool active = 16 * NG * wv < R;  // waves without rows only help moving blocks
+    // A single-token sequence whose scores are wanted: wave 0 keeps its heads' probabilities and per-tile maxima in LDS
+    // and the workgroup writes them out behind the loop.  (A store inside the loop would make every wait for a block
+    // fetch a wait for all of them: loads and stores share a counter and complete out of order with respect to each
+    // other.)  The host keeps such items at single_item_max_tiles(G) tiles.
+    constexpr bool STASH = !U8 && !XATT && !DMA && NG == 1;
+    __shared__ __align__(16) uint8_t pkeep[STASH ? SINGLE_STASH_BYTES : 16];
+    bool emit = false;
+    if constexpr (STASH) emit = a.p_out != nullptr && a.single_idx[b] >= 0;
 
     // ---- the pieces of work on a block ---------------------------------------------------------------------
     // S^T = K . Q^T for both row groups (block number jk) and O^T += V^T . P^T (block number jv), issued as one
@@ -549,6 +557,22 @@ void pa_prefill16_kernel(PrefillArgs a) {
                     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
                     const h2 h = __builtin_bit_cast(h2, hi);
                     pl[gi][jj] = pack2<DT>(p[2 * jj] - (float)h[0], p[2 * jj + 1] - (float)h[1]);
+                }
+                if constexpr (STASH) {
+                    if (emit && gi == 0) {
+                        // (head and token group of the lane from an opaque copy of the thread id: kept in registers of
+                        // their own across the loop they would cost this variant a spill; pair by pair for the same
+                        // reason)  LDS image: [tile of the item][head of the group][32 tokens], then [tile][head] maxima
+                        int te_ = threadIdx.x;
+                        asm volatile("" : "+v"(te_));
+                        const int ne = te_ & 15, ge = (te_ >> 4) & 3;
+                        if (ne < G) {
+                            uint8_t* at = pkeep + ((j * G + ne) * TOK + 4 * ge + 16 * (jj >> 1) + 2 * (jj & 1)) * 2;
+                            *reinterpret_cast<uint32_t*>(at) = pack2<DT_F16>(p[2 * jj], p[2 * jj + 1]);
+                            if (jj == 0 && ge == 0)
+                                *reinterpret_cast<float*>(pkeep + single_item_max_tiles(G) * G * TOK * 2 + (j * G + ne) * 4) = m_safe;
+                        }
+                    }
                 }
             }
             l_part[gi] = l_part[gi] * corr[gi] + psum;
@@ -752,6 +776,10 @@ void pa_prefill16_kernel(PrefillArgs a) {
     // alive across the loop it costs the variants that sit at their register limit a spill
     int ge = threadIdx.x;
     asm volatile("" : "+v"(ge));
+    if constexpr (STASH) {  // ... and the row's id, for the same reason (one row group per wave)
+        const int rho = min(16 * (ge >> 6) + (ge & 15), R - 1);
+        row_id[0] = (t0 + q0 + rho / G) * Hq + hkv * G + rho % G;
+    }
     ge = (ge >> 4) & 3;
 #pragma unroll
     for (int gi = 0; gi < NG; ++gi) {
@@ -784,6 +812,22 @@ void pa_prefill16_kernel(PrefillArgs a) {
                 a.part_ml[2 * slot] = m_run[gi];
                 a.part_ml[2 * slot + 1] = l;
             }
+        }
+    }
+    if constexpr (STASH) {
+        if (emit) {  // (uniform) behind the rows, with their registers free: the item's probabilities and maxima: LDS -> [tile][Hq][32] / [tile][Hq]
+            __syncthreads();
+            const long tile0 = tile_max_offset(st.score_offsets[b], b) + tb;
+            int te_ = threadIdx.x;
+            asm volatile("" : "+v"(te_));
+            for (int i = te_; i < cnt * G * (TOK / 8); i += NT) {  // 16-byte pieces
+                const int piece = i % (TOK / 8), h = (i / (TOK / 8)) % G, jt = i / (TOK / 8) / G;
+                *reinterpret_cast<u4v*>(a.p_out + ((tile0 + jt) * Hq + hkv * G + h) * TOK + piece * 8) =
+                    *reinterpret_cast<const u4v*>(pkeep + ((jt * G + h) * TOK + piece * 8) * 2);
+            }
+            for (int i = te_; i < cnt * G; i += NT)
+                a.tile_max[(tile0 + i / G) * Hq + hkv * G + i % G] =
+                    *reinterpret_cast<const float*>(pkeep + single_item_max_tiles(G) * G * TOK * 2 + i * 4);
         }
     }
 }
@@ -852,7 +896,70 @@ __global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(PrefillArgs a) 
     }
 }
 
+// Scores of single-token sequences from the probabilities the matrix kernel left: score[pos] = sum over heads of
+// p[h][pos] * 2^(tile maximum - final maximum) / denominator.  One workgroup per (2048 positions, sequence); a thread
+// takes eight positions of one tile; heads are added in ascending order (fixed order, no atomics), four heads' loads
+// in flight at a time.
+__global__ __launch_bounds__(256) void pa_single_scores_kernel(PrefillArgs a, const int32_t* __restrict__ seq_list,
+                                                               float* __restrict__ scores) {
+    extern __shared__ float s_ml[];  // [Hq][2]: final maximum (log2 domain), 1 / denominator
+    const StepDev& st = a.st;
+    const int b = seq_list[blockIdx.y];
+    const int t = st.subsequence_begins[b];
+    const int kv_len = st.past_lens[b] + 1;
+    const int first = st.sliding_window > 0 ? max(0, kv_len - st.sliding_window) : 0;
+    const int W = st.score_window[b];
+    const long so = st.score_offsets[b];
+    float* out = scores + so;
+    const int Hq = a.sh.Hq;
+    for (int h = threadIdx.x; h < Hq; h += 256) {
+        const float2 ml = *reinterpret_cast<const float2*>(a.final_ml + 2 * ((long)t * Hq + h));
+        s_ml[2 * h] = ml.x * LOG2E;
+        s_ml[2 * h + 1] = ml.y > 0.0f ? 1.0f / ml.y : 0.0f;
+    }
+    __syncthreads();
+    const long tg0 = tile_max_offset(so, b) * (long)Hq;  // [tile][head] of the sequence's first tile
+    const _Float16* p = a.p_out + tg0 * TOK;
+    const float* tmax = a.tile_max + tg0;
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    for (int pos = (blockIdx.x * 256 + threadIdx.x) * 8; pos < kv_len; pos += gridDim.x * 2048) {
+        float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (W > 0 && pos + 7 >= first) {  // (tiles in front of the window's were not walked)
+            const long th0 = (long)(pos >> 5) * Hq;
+            for (int h0 = 0; h0 < Hq; h0 += 4) {
+                h8 v[4];
+                float f[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = min(h0 + i, Hq - 1);
+                    v[i] = *reinterpret_cast<const h8*>(p + (th0 + h) * TOK + (pos & 31));
+                    f[i] = tmax[th0 + h];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = min(h0 + i, Hq - 1);
+                    const float fac = h0 + i < Hq ? __builtin_amdgcn_exp2f(f[i] - s_ml[2 * h]) * s_ml[2 * h + 1] : 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) s[e] += (float)v[i][e] * fac;
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (pos + e < kv_len) out[pos + e] = pos + e >= first ? s[e] : 0.0f;
+    }
+}
+
 }  // namespace
+
+hipError_t launch_single_scores(hipStream_t s, const PrefillArgs& a, const int32_t* seq_list, int n_seqs, float* scores,
+                                int max_kv_len) {
+    if (n_seqs <= 0) return hipSuccess;
+    if (n_seqs > 65535) return hipErrorInvalidValue;
+    dim3 grid((unsigned)min(ceil_div(max_kv_len, 2048), 64), (unsigned)n_seqs);
+    hipLaunchKernelGGL(pa_single_scores_kernel, grid, dim3(256), (size_t)a.sh.Hq * 2 * sizeof(float), s, a, seq_list, scores);
+    return hipGetLastError();
+}
 
 template <int D, int DT, int QDT, bool U8>
 static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1) {

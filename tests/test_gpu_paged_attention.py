@@ -167,6 +167,14 @@ def test_decode_u8_kernel_shapes(pkg, dev, name, args, kw):
     # many long single-token sequences next to two short chunks: their work items are listed between the chunks' items
     ("pf16_bf16_interleaved_items", (28, 4, 128, 32, "bf16", "bf16",
                                      [100, 0] + [900 + 37 * i for i in range(14)], [64, 40] + [1] * 14), {}),
+    # long single-token sequences next to chunks, scores wanted: their items keep the probabilities in LDS (several
+    # items per sequence) and a small kernel forms the scores; windows of 0 and 1 rows, a sliding window, G = 16
+    ("pf16_bf16_g7_long_singles", (28, 4, 128, 32, "bf16", "bf16", [0, 5000, 4097, 1375, 1376, 1377, 9000],
+                                   [100, 1, 1, 1, 1, 1, 1]), {"score_aggregation_window": [4, 1, 0, 1, 1, 1, 1]}),
+    ("pf16_f16_g16_long_singles_window", (16, 1, 128, 32, "f16", "f16", [64, 3000, 700, 6000], [40, 1, 1, 1]),
+     {"sliding_window": 2500}),
+    ("pf16_f16_d64_g1_long_singles", (4, 4, 64, 32, "f16", "f16", [10, 7000, 33], [70, 1, 1]), {}),
+    ("pf16_bf16_block16_long_singles", (8, 2, 128, 16, "bf16", "bf16", [0, 5000, 2049], [50, 1, 1]), {}),
     ("pf16_f16_interleaved_items_window", (8, 2, 64, 32, "f16", "f16",
                                            [300] + [700 + 11 * i for i in range(9)], [50] + [1] * 9),
      {"sliding_window": 600, "score_aggregation_window": [5] + [1] * 9}),

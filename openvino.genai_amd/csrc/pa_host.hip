@@ -430,6 +430,15 @@ void plan_items(pa_ctx* ctx) {
         for (int32_t i = 0; i < t.nq; ++i) tok_ns[sb[t.b] + t.q0 + i] = ns;
         max_split = std::max(max_split, ns);
     }
+    // Workgroups start in list order and a CU slot works through two or three of them in a launch: the dense items of
+    // multi-token sequences are listed longest first (within the wide and the narrow group), so that no long item
+    // starts last and finishes alone.
+    {
+        auto longer = [](const pa::PrefillItem& x, const pa::PrefillItem& y) { return x.te - x.tb > y.te - y.tb; };
+        const int32_t n_multi = (int32_t)items.size() - ctx->n_sparse - ctx->n_single;
+        std::stable_sort(items.begin(), items.begin() + ctx->n_wide, longer);
+        std::stable_sort(items.begin() + ctx->n_wide, items.begin() + n_multi, longer);
+    }
     PA_REQUIRE(longest_sparse <= 128, PA_UNKNOWN_EXCEPTION, "a block-sparse work item walks more than 128 KV blocks");
     // A mixed step over a 16-bit cache runs the single-token items (bandwidth-bound) and the chunk items
     // (matrix-bound) in one launch of one kernel variant.  Workgroups start in list order, so the two kinds only share

@@ -128,6 +128,7 @@ struct pa_ctx {
     std::vector<int32_t> h_dec16;     // single-token sequences of a 16-bit-cache step (also listed as matrix-kernel items)
     DevBuf dec16_list;
     DevBuf tile_max;   // per (head, 32-token tile) maxima of single-token sequences handled by the matrix kernel
+    bool dec_in_order = false, dec16_in_order = false;  // the lists hold 0 .. B-1 in order: every sequence, none moved
     bool stash_ok = false;  // the step's single-token items are short enough to keep their probabilities in LDS
     int32_t n_items = 0, n_wide = 0, max_split = 1;
     size_t tok_nsplit_off = 0;
@@ -466,6 +467,21 @@ void plan_items(pa_ctx* ctx) {
             items.swap(mixed);
         }
     }
+    // The decode kernels' workgroups start in list order too: longest contexts first (equal lengths keep their order, and
+    // a list that is 0, 1, 2, ... is not passed at all)
+    {
+        auto longer = [&](int32_t x, int32_t y) { return past[x] > past[y]; };
+        std::stable_sort(ctx->h_dec.begin(), ctx->h_dec.end(), longer);
+        std::stable_sort(ctx->h_dec16.begin(), ctx->h_dec16.end(), longer);
+        auto identity = [&](const std::vector<int32_t>& v) {
+            if ((int32_t)v.size() != B) return false;
+            for (int32_t i = 0; i < B; ++i)
+                if (v[i] != i) return false;
+            return true;
+        };
+        ctx->dec_in_order = identity(ctx->h_dec);
+        ctx->dec16_in_order = identity(ctx->h_dec16);
+    }
     ctx->x_keep_words = 1 + longest_sparse;  // entries of a work item's block list
     ctx->n_items = (int32_t)items.size();
     ctx->max_split = max_split;
@@ -589,7 +605,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.value = static_cast<const uint16_t*>(io->value);
         a.fuse_append = fuse_append ? 1 : 0;
         a.n_seqs = (int32_t)ctx->h_dec.size();
-        a.seq_list = a.n_seqs == ctx->B ? nullptr : ctx->dec_list.as<int32_t>();
+        a.seq_list = ctx->dec_in_order ? nullptr : ctx->dec_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
         const DecodeWs ws = decode_workspace(ctx, rows, a.nsplit, io->scores != nullptr, static_ws);
         a.query = static_cast<const uint16_t*>(io->query);
@@ -616,7 +632,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         plan_decode_u8(ctx, io->scores != nullptr, &a.nsplit, &a.max_tiles, &ctx->h_dec16);
         a.waves = 4;
         a.n_seqs = (int32_t)ctx->h_dec16.size();
-        a.seq_list = a.n_seqs == ctx->B ? nullptr : ctx->dec16_list.as<int32_t>();
+        a.seq_list = ctx->dec16_in_order ? nullptr : ctx->dec16_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
         const DecodeWs ws = decode_workspace(ctx, rows, a.nsplit, io->scores != nullptr, static_ws);
         a.query = static_cast<const uint16_t*>(io->query);

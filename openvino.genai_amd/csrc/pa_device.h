@@ -289,9 +289,69 @@ __host__ __device__ inline int single_item_max_tiles(int G) { return SINGLE_STAS
 // Tiles of the sequences of a step, one after the other: a sequence of kv_len positions takes ceil(kv_len / 32).
 __host__ __device__ inline long tile_max_offset(long score_offset, int b) { return (score_offset >> 5) + b; }
 __host__ __device__ inline long tile_max_count(long total_scores, int B) { return (total_scores >> 5) + B + 1; }
-// Scores of the listed single-token sequences from what the matrix kernel left (after its merge kernel).
-hipError_t launch_single_scores(hipStream_t s, const PrefillArgs& a, const int32_t* seq_list, int n_seqs, float* scores,
-                                int max_kv_len);
+// Scores of single-token sequences from the probabilities the matrix kernel left (after its merge kernel):
+// score[pos] = sum over heads of p[h][pos] * 2^(tile maximum - final maximum) / denominator.  Runs as extra workgroups
+// of the score replay's launch (rows of the grid behind the sequences', one per listed sequence; `gx` workgroups of
+// 2048 positions each per row): both wait for the same merge, both are short and bound by latency.
+struct SingleScores {
+    const _Float16* p_out;   // null: no such rows
+    const float* tile_max;
+    const int32_t* seq_list;
+    int32_t n_seqs, gx;
+};
+#if defined(__HIPCC__)
+__device__ __forceinline__ void single_scores_rows(const StepDev& st, const Shape& sh, const SingleScores& ss,
+                                                   const float* __restrict__ final_ml, float* __restrict__ scores,
+                                                   const int row, const int bx) {
+    __shared__ float s_ml[2 * 256];  // [Hq][2]: final maximum (log2 domain), 1 / denominator
+    constexpr float LOG2E_ = 1.4426950408889634f;
+    if (bx >= ss.gx) return;
+    const int b = ss.seq_list[row];
+    const int t = st.subsequence_begins[b];
+    const int kv_len = st.past_lens[b] + 1;
+    const int first = st.sliding_window > 0 ? max(0, kv_len - st.sliding_window) : 0;
+    const int W = st.score_window[b];
+    const long so = st.score_offsets[b];
+    float* out = scores + so;
+    const int Hq = sh.Hq;
+    for (int h = threadIdx.x; h < Hq; h += 256) {
+        const float2 ml = *reinterpret_cast<const float2*>(final_ml + 2 * ((long)t * Hq + h));
+        s_ml[2 * h] = ml.x * LOG2E_;
+        s_ml[2 * h + 1] = ml.y > 0.0f ? 1.0f / ml.y : 0.0f;
+    }
+    __syncthreads();
+    const long tg0 = tile_max_offset(so, b) * (long)Hq;  // [tile][head] of the sequence's first tile
+    const _Float16* p = ss.p_out + tg0 * 32;
+    const float* tmax = ss.tile_max + tg0;
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    for (int pos = (bx * 256 + threadIdx.x) * 8; pos < kv_len; pos += ss.gx * 2048) {
+        float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (W > 0 && pos + 7 >= first) {  // (tiles in front of the window's were not walked)
+            const long th0 = (long)(pos >> 5) * Hq;
+            for (int h0 = 0; h0 < Hq; h0 += 4) {  // heads in ascending order (fixed order, no atomics), four in flight
+                h8 v[4];
+                float f[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = min(h0 + i, Hq - 1);
+                    v[i] = *reinterpret_cast<const h8*>(p + (th0 + h) * 32 + (pos & 31));
+                    f[i] = tmax[th0 + h];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = min(h0 + i, Hq - 1);
+                    const float fac = h0 + i < Hq ? __builtin_amdgcn_exp2f(f[i] - s_ml[2 * h]) * s_ml[2 * h + 1] : 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) s[e] += (float)v[i][e] * fac;
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (pos + e < kv_len) out[pos + e] = pos + e >= first ? s[e] : 0.0f;
+    }
+}
+#endif
 hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, int kv_dtype, hipEvent_t ev0,
                             hipEvent_t ev1);
 
@@ -335,7 +395,7 @@ hipError_t launch_rotate(hipStream_t s, void* key_cache, int kv_dtype, const Sha
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
                                 float* final_ml, float* scores, int32_t max_kv_len, int single_token_too,
-                                const XattDev& xd);
+                                const XattDev& xd, const SingleScores& ss);
 
 // Block diversity of the evictable area (pa_rkv_diversity.hip).
 struct RkvDivSeq {          // one sequence whose diversity is computed

@@ -724,15 +724,20 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         if (!use_decode && !use_decode16) ctx->nsplit = ctx->max_split;
         HIP_CHECK(pa::launch_prefill16(ctx->stream, a, c.query_dtype, c.kv_cache_dtype, ev0, ev1));
         ctx->timed = ctx->profiling;
-        if (hand_over)
-            HIP_CHECK(pa::launch_single_scores(ctx->stream, a, ctx->dec16_list.as<int32_t>(), (int)ctx->h_dec16.size(),
-                                               io->scores, ctx->max_kv));
-        // scores of the multi-token sequences (and of single-token ones that were work items of this kernel and left
-        // nothing for the score kernel): replay
-        if (io->scores && !(use_decode16 && ctx->n_single == ctx->n_items))
+        // scores of the multi-token sequences (and of single-token ones that were work items of this kernel and kept
+        // nothing for the score rows): replay; the kept probabilities become scores in extra rows of the same launch
+        if (io->scores && !(use_decode16 && ctx->n_single == ctx->n_items)) {
+            pa::SingleScores ss{};
+            if (hand_over) {
+                ss.p_out = a.p_out;
+                ss.tile_max = a.tile_max;
+                ss.seq_list = ctx->dec16_list.as<int32_t>();
+                ss.n_seqs = (int32_t)ctx->h_dec16.size();
+            }
             HIP_CHECK(pa::launch_scores_replay(ctx->stream, ctx->dev, a.sh, c.query_dtype, c.kv_cache_dtype, io->query,
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
-                                               decode_u8_shape(c) || use_decode16 || hand_over ? 0 : 1, a.xatt));
+                                               decode_u8_shape(c) || use_decode16 || hand_over ? 0 : 1, a.xatt, ss));
+        }
     }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;

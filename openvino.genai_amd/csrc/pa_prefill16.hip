@@ -832,46 +832,54 @@ void pa_prefill16_kernel(PrefillArgs a) {
     }
 }
 
-// Rows whose context was cut into several ranges: fold the partials (maxima in the log2 domain).
+// Rows whose context was cut into several ranges: fold the partials (maxima in the log2 domain).  Sixteen lanes per
+// row, D / 16 channels each (16-byte loads), four rows per wave; ranges are folded in ascending order.
 template <int D, int DT>
 __global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(PrefillArgs a) {
-    constexpr int EPL = D / 64;
-    const int lane = threadIdx.x & 63;
-    const long idx = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (idx >= (long)a.n_merge * a.sh.Hq) return;
+    constexpr int EPL = D / 16;
+    const int l16 = threadIdx.x & 15;
+    long idx = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const long n_rows = (long)a.n_merge * a.sh.Hq;
+    const bool live = idx < n_rows;
+    idx = min(idx, n_rows - 1);  // (surplus groups repeat the last row and store nothing: no divergence around the shuffles)
     const int tok = a.merge_tokens[idx / a.sh.Hq];
     const long row = (long)tok * a.sh.Hq + idx % a.sh.Hq;
-    if (a.skip_single && a.single_idx[a.st.token_seq[tok]] >= 0) return;  // another kernel's rows
+    const bool mine = live && !(a.skip_single && a.single_idx[a.st.token_seq[tok]] >= 0);  // (else another kernel's row)
     const int ns = a.tok_nsplit[tok];
     float acc[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
     float M, L;
-    if (ns <= WAVE) {
-        // lane s holds range s: one round of loads instead of a dependent chain
-        const float2 ml = lane < ns ? *reinterpret_cast<const float2*>(a.part_ml + 2 * (row * a.max_split + lane))
-                                    : make_float2(-INFINITY, 0.0f);
-        M = wave_max(ml.x);
+    if (ns <= 16) {
+        // lane s of the group holds range s: one round of loads instead of a dependent chain
+        const float2 ml = l16 < ns ? *reinterpret_cast<const float2*>(a.part_ml + 2 * (row * a.max_split + l16))
+                                   : make_float2(-INFINITY, 0.0f);
+        M = ml.x;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 16));
         const float f_mine = ml.x == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml.x - M);
-        L = wave_sum(ml.y * f_mine);
+        L = ml.y * f_mine;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) L += __shfl_xor(L, o, 16);
         // four ranges per round, loaded unconditionally (indices clamped, surplus ones weighted zero) so that
         // a round's loads are in flight together
         for (int s0 = 0; s0 < ns; s0 += 4) {
-            float ms[4], v[4][EPL];
+            float f[4];
+            f4 v[4][EPL / 4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const long slot = row * a.max_split + min(s0 + j, ns - 1);
-                ms[j] = a.part_ml[2 * slot];  // same address in every lane: one broadcast load
-                const float* pa = a.part_acc + slot * D + lane * EPL;
+                f[j] = __shfl(f_mine, min(s0 + j, ns - 1), 16);
+                if (s0 + j >= ns) f[j] = 0.0f;
+                const f4* pa = reinterpret_cast<const f4*>(a.part_acc + slot * D + l16 * EPL);
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) v[j][e] = pa[e];
+                for (int e = 0; e < EPL / 4; ++e) v[j][e] = pa[e];
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float f = (s0 + j >= ns || ms[j] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[j] - M);
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) acc[e] = fmaf(f == 0.0f ? 0.0f : v[j][e], f, acc[e]);  // fully masked ranges hold nothing
-            }
+                for (int e = 0; e < EPL; ++e)
+                    acc[e] = fmaf(f[j] == 0.0f ? 0.0f : v[j][e / 4][e % 4], f[j], acc[e]);  // fully masked ranges hold nothing
         }
     } else {
         M = -INFINITY;
@@ -884,82 +892,25 @@ __global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(PrefillArgs a) 
             const float f = __builtin_amdgcn_exp2f(ms - M);
             L += a.part_ml[2 * slot + 1] * f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + lane * EPL + e] * f;
+            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + l16 * EPL + e] * f;
         }
     }
+    if (!mine) return;
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    uint32_t o[EPL / 2];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) a.out[row * D + lane * EPL + e] = store16<DT>(acc[e] * inv);
-    if (lane == 0) {
+    for (int e = 0; e < EPL / 2; ++e)
+        o[e] = (uint32_t)store16<DT>(acc[2 * e] * inv) | ((uint32_t)store16<DT>(acc[2 * e + 1] * inv) << 16);
+    uint16_t* dst = a.out + row * D + l16 * EPL;
+    if constexpr (EPL == 8) *reinterpret_cast<u4v*>(dst) = u4v{o[0], o[1], o[2], o[3]};
+    else *reinterpret_cast<uint2*>(dst) = make_uint2(o[0], o[1]);
+    if (l16 == 0) {
         a.final_ml[2 * row] = M * LN2;
         a.final_ml[2 * row + 1] = L;
     }
 }
 
-// Scores of single-token sequences from the probabilities the matrix kernel left: score[pos] = sum over heads of
-// p[h][pos] * 2^(tile maximum - final maximum) / denominator.  One workgroup per (2048 positions, sequence); a thread
-// takes eight positions of one tile; heads are added in ascending order (fixed order, no atomics), four heads' loads
-// in flight at a time.
-__global__ __launch_bounds__(256) void pa_single_scores_kernel(PrefillArgs a, const int32_t* __restrict__ seq_list,
-                                                               float* __restrict__ scores) {
-    extern __shared__ float s_ml[];  // [Hq][2]: final maximum (log2 domain), 1 / denominator
-    const StepDev& st = a.st;
-    const int b = seq_list[blockIdx.y];
-    const int t = st.subsequence_begins[b];
-    const int kv_len = st.past_lens[b] + 1;
-    const int first = st.sliding_window > 0 ? max(0, kv_len - st.sliding_window) : 0;
-    const int W = st.score_window[b];
-    const long so = st.score_offsets[b];
-    float* out = scores + so;
-    const int Hq = a.sh.Hq;
-    for (int h = threadIdx.x; h < Hq; h += 256) {
-        const float2 ml = *reinterpret_cast<const float2*>(a.final_ml + 2 * ((long)t * Hq + h));
-        s_ml[2 * h] = ml.x * LOG2E;
-        s_ml[2 * h + 1] = ml.y > 0.0f ? 1.0f / ml.y : 0.0f;
-    }
-    __syncthreads();
-    const long tg0 = tile_max_offset(so, b) * (long)Hq;  // [tile][head] of the sequence's first tile
-    const _Float16* p = a.p_out + tg0 * TOK;
-    const float* tmax = a.tile_max + tg0;
-    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-    for (int pos = (blockIdx.x * 256 + threadIdx.x) * 8; pos < kv_len; pos += gridDim.x * 2048) {
-        float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        if (W > 0 && pos + 7 >= first) {  // (tiles in front of the window's were not walked)
-            const long th0 = (long)(pos >> 5) * Hq;
-            for (int h0 = 0; h0 < Hq; h0 += 4) {
-                h8 v[4];
-                float f[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int h = min(h0 + i, Hq - 1);
-                    v[i] = *reinterpret_cast<const h8*>(p + (th0 + h) * TOK + (pos & 31));
-                    f[i] = tmax[th0 + h];
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int h = min(h0 + i, Hq - 1);
-                    const float fac = h0 + i < Hq ? __builtin_amdgcn_exp2f(f[i] - s_ml[2 * h]) * s_ml[2 * h + 1] : 0.0f;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) s[e] += (float)v[i][e] * fac;
-                }
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-            if (pos + e < kv_len) out[pos + e] = pos + e >= first ? s[e] : 0.0f;
-    }
-}
-
 }  // namespace
-
-hipError_t launch_single_scores(hipStream_t s, const PrefillArgs& a, const int32_t* seq_list, int n_seqs, float* scores,
-                                int max_kv_len) {
-    if (n_seqs <= 0) return hipSuccess;
-    if (n_seqs > 65535) return hipErrorInvalidValue;
-    dim3 grid((unsigned)min(ceil_div(max_kv_len, 2048), 64), (unsigned)n_seqs);
-    hipLaunchKernelGGL(pa_single_scores_kernel, grid, dim3(256), (size_t)a.sh.Hq * 2 * sizeof(float), s, a, seq_list, scores);
-    return hipGetLastError();
-}
 
 template <int D, int DT, int QDT, bool U8>
 static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1) {
@@ -997,7 +948,7 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
     if (ev1) (void)hipEventRecord(ev1, s);
     if (a.n_merge > 0) {
         const long rows = (long)a.n_merge * a.sh.Hq;
-        hipLaunchKernelGGL((pa_prefill16_merge_kernel<D, QDT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((pa_prefill16_merge_kernel<D, QDT>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
     }
     return hipGetLastError();
 }

@@ -57,11 +57,15 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
                                                              const int32_t* __restrict__ block_indices,
                                                              const float* __restrict__ final_ml,
                                                              float* __restrict__ scores, int single_token_too,
-                                                             XattDev xd) {
+                                                             XattDev xd, SingleScores ss) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     constexpr int KS = D / 32;
     constexpr int CROWB = U8 ? D + 8 : D * 2;
     constexpr float CODE_UNIT = 16777216.0f;  // a code byte read as f16 is code * 2^-24
+    if ((int)blockIdx.y >= st.B) {  // the rows behind the sequences': single-token sequences whose probabilities were kept
+        single_scores_rows(st, sh, ss, final_ml, scores, (int)blockIdx.y - st.B, (int)blockIdx.x);
+        return;
+    }
     const int b = blockIdx.y;
     const int t0 = st.subsequence_begins[b];
     const int q_len = st.subsequence_begins[b + 1] - t0;
@@ -200,15 +204,19 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
                                 float* final_ml, float* scores, int32_t max_kv_len, int single_token_too,
-                                const XattDev& xd) {
+                                const XattDev& xd, const SingleScores& ss_in) {
     if (st.B == 0 || max_kv_len <= 0) return hipSuccess;
-    const dim3 grid((unsigned)ceil_div(max_kv_len, 4 * TN), (unsigned)st.B), block(256);
+    SingleScores ss = ss_in;
+    if (!ss.p_out) ss.n_seqs = 0;
+    if (sh.Hq > 256 || st.B + ss.n_seqs > 65535) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)ceil_div(max_kv_len, 4 * TN), (unsigned)(st.B + ss.n_seqs)), block(256);
+    ss.gx = min(ceil_div(max_kv_len, 2048), 64);  // (at most the grid's width: 2048 > 4 * TN)
     auto q = reinterpret_cast<const uint16_t*>(query);
     auto k = reinterpret_cast<const uint8_t*>(key_cache);
 #define PA_REPLAY(DD, DT, Q, U8)                                                                               \
     {                                                                                                          \
         hipLaunchKernelGGL((pa_scores_mfma_kernel<DD, DT, Q, U8>), grid, block, 0, s, st, sh, q, k,            \
-                           block_indices, final_ml, scores, single_token_too, xd);                             \
+                           block_indices, final_ml, scores, single_token_too, xd, ss);                         \
         return hipGetLastError();                                                                              \
     }
     if (sh.bs != 32 && sh.bs != 16) return hipErrorInvalidValue;

@@ -328,17 +328,18 @@ __device__ __forceinline__ void single_scores_rows(const StepDev& st, const Shap
         float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         if (W > 0 && pos + 7 >= first) {  // (tiles in front of the window's were not walked)
             const long th0 = (long)(pos >> 5) * Hq;
-            for (int h0 = 0; h0 < Hq; h0 += 4) {  // heads in ascending order (fixed order, no atomics), four in flight
-                h8 v[4];
-                float f[4];
+            constexpr int HU = 8;  // heads whose loads are in flight together
+            for (int h0 = 0; h0 < Hq; h0 += HU) {  // heads in ascending order (fixed order, no atomics)
+                h8 v[HU];
+                float f[HU];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < HU; ++i) {
                     const int h = min(h0 + i, Hq - 1);
                     v[i] = *reinterpret_cast<const h8*>(p + (th0 + h) * 32 + (pos & 31));
                     f[i] = tmax[th0 + h];
                 }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < HU; ++i) {
                     const int h = min(h0 + i, Hq - 1);
                     const float fac = h0 + i < Hq ? __builtin_amdgcn_exp2f(f[i] - s_ml[2 * h]) * s_ml[2 * h + 1] : 0.0f;
 #pragma unroll
@@ -394,8 +395,8 @@ hipError_t launch_rotate(hipStream_t s, void* key_cache, int kv_dtype, const Sha
 // Scores by replaying the last W query rows of every sequence against the positions they see (needs final_ml).
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
-                                float* final_ml, float* scores, int32_t max_kv_len, int single_token_too,
-                                const XattDev& xd, const SingleScores& ss);
+                                float* final_ml, float* scores, int32_t max_kv_len, const int32_t* seq_list,
+                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss);
 
 // Block diversity of the evictable area (pa_rkv_diversity.hip).
 struct RkvDivSeq {          // one sequence whose diversity is computed

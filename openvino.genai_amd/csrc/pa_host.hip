@@ -127,6 +127,8 @@ struct pa_ctx {
     std::vector<int32_t> h_dec;
     std::vector<int32_t> h_dec16;     // single-token sequences of a 16-bit-cache step (also listed as matrix-kernel items)
     DevBuf dec16_list;
+    std::vector<int32_t> h_multi;     // sequences that schedule more than one token
+    DevBuf multi_list;
     DevBuf tile_max;   // per (head, 32-token tile) maxima of single-token sequences handled by the matrix kernel
     bool dec_in_order = false, dec16_in_order = false;  // the lists hold 0 .. B-1 in order: every sequence, none moved
     bool stash_ok = false;  // the step's single-token items are short enough to keep their probabilities in LDS
@@ -502,6 +504,17 @@ void plan_items(pa_ctx* ctx) {
     HIP_CHECK(hipMemcpyAsync(ctx->items.p, items.data(), item_bytes, hipMemcpyHostToDevice, ctx->stream));
     HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(ctx->items.p) + item_bytes, tok_ns.data(),
                              tok_ns.size() * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    // the sequences a score replay has rows for: those with more than one token, longest context first
+    ctx->h_multi.clear();
+    for (int32_t b = 0; b < B; ++b)
+        if (sb[b + 1] - sb[b] > 1) ctx->h_multi.push_back(b);
+    std::stable_sort(ctx->h_multi.begin(), ctx->h_multi.end(),
+                     [&](int32_t x, int32_t y) { return past[x] + sb[x + 1] - sb[x] > past[y] + sb[y + 1] - sb[y]; });
+    if (!ctx->h_multi.empty()) {
+        ctx->multi_list.reserve(ctx->h_multi.size() * sizeof(int32_t));
+        HIP_CHECK(hipMemcpyAsync(ctx->multi_list.p, ctx->h_multi.data(), ctx->h_multi.size() * sizeof(int32_t),
+                                 hipMemcpyHostToDevice, ctx->stream));
+    }
     if (!ctx->h_dec16.empty()) {
         ctx->dec16_list.reserve(ctx->h_dec16.size() * sizeof(int32_t));
         HIP_CHECK(hipMemcpyAsync(ctx->dec16_list.p, ctx->h_dec16.data(), ctx->h_dec16.size() * sizeof(int32_t),
@@ -734,9 +747,12 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                 ss.seq_list = ctx->dec16_list.as<int32_t>();
                 ss.n_seqs = (int32_t)ctx->h_dec16.size();
             }
+            // (without the single-token sequences the launch has rows for the listed multi-token sequences only)
+            const bool singles_too = !(decode_u8_shape(c) || use_decode16 || hand_over);
             HIP_CHECK(pa::launch_scores_replay(ctx->stream, ctx->dev, a.sh, c.query_dtype, c.kv_cache_dtype, io->query,
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
-                                               decode_u8_shape(c) || use_decode16 || hand_over ? 0 : 1, a.xatt, ss));
+                                               singles_too ? nullptr : ctx->multi_list.as<int32_t>(),
+                                               singles_too ? ctx->B : (int32_t)ctx->h_multi.size(), a.xatt, ss));
         }
     }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
@@ -793,6 +809,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->pf_part_ml.release();
     ctx->dec_list.release();
     ctx->dec16_list.release();
+    ctx->multi_list.release();
     ctx->tile_max.release();
     ctx->trig_lut.release();
     ctx->rot_args.release();

@@ -56,20 +56,20 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
                                                              const uint8_t* __restrict__ key_cache,
                                                              const int32_t* __restrict__ block_indices,
                                                              const float* __restrict__ final_ml,
-                                                             float* __restrict__ scores, int single_token_too,
+                                                             float* __restrict__ scores,
+                                                             const int32_t* __restrict__ seq_list, int n_seqs,
                                                              XattDev xd, SingleScores ss) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     constexpr int KS = D / 32;
     constexpr int CROWB = U8 ? D + 8 : D * 2;
     constexpr float CODE_UNIT = 16777216.0f;  // a code byte read as f16 is code * 2^-24
-    if ((int)blockIdx.y >= st.B) {  // the rows behind the sequences': single-token sequences whose probabilities were kept
-        single_scores_rows(st, sh, ss, final_ml, scores, (int)blockIdx.y - st.B, (int)blockIdx.x);
+    if ((int)blockIdx.y >= n_seqs) {  // the rows behind the sequences': single-token sequences whose probabilities were kept
+        single_scores_rows(st, sh, ss, final_ml, scores, (int)blockIdx.y - n_seqs, (int)blockIdx.x);
         return;
     }
-    const int b = blockIdx.y;
+    const int b = seq_list ? seq_list[blockIdx.y] : (int)blockIdx.y;  // the listed sequences, or all of the step's
     const int t0 = st.subsequence_begins[b];
     const int q_len = st.subsequence_begins[b + 1] - t0;
-    if (q_len <= 1 && !single_token_too) return;
     const int past = st.past_lens[b];
     const int kv_len = past + q_len;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -203,20 +203,20 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
 
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
-                                float* final_ml, float* scores, int32_t max_kv_len, int single_token_too,
-                                const XattDev& xd, const SingleScores& ss_in) {
-    if (st.B == 0 || max_kv_len <= 0) return hipSuccess;
+                                float* final_ml, float* scores, int32_t max_kv_len, const int32_t* seq_list,
+                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss_in) {
     SingleScores ss = ss_in;
     if (!ss.p_out) ss.n_seqs = 0;
-    if (sh.Hq > 256 || st.B + ss.n_seqs > 65535) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)ceil_div(max_kv_len, 4 * TN), (unsigned)(st.B + ss.n_seqs)), block(256);
+    if (n_seqs + ss.n_seqs == 0 || max_kv_len <= 0) return hipSuccess;
+    if (sh.Hq > 256 || n_seqs + ss.n_seqs > 65535) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)ceil_div(max_kv_len, 4 * TN), (unsigned)(n_seqs + ss.n_seqs)), block(256);
     ss.gx = min(ceil_div(max_kv_len, 2048), 64);  // (at most the grid's width: 2048 > 4 * TN)
     auto q = reinterpret_cast<const uint16_t*>(query);
     auto k = reinterpret_cast<const uint8_t*>(key_cache);
 #define PA_REPLAY(DD, DT, Q, U8)                                                                               \
     {                                                                                                          \
         hipLaunchKernelGGL((pa_scores_mfma_kernel<DD, DT, Q, U8>), grid, block, 0, s, st, sh, q, k,            \
-                           block_indices, final_ml, scores, single_token_too, xd, ss);                         \
+                           block_indices, final_ml, scores, seq_list, n_seqs, xd, ss);                         \
         return hipGetLastError();                                                                              \
     }
     if (sh.bs != 32 && sh.bs != 16) return hipErrorInvalidValue;

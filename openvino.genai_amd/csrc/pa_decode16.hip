@@ -70,6 +70,10 @@ template <int D, int DT, int BS>
 __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
     constexpr int WAVES = 4;
     constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile (with two, each holds one row group)
+    // BS = 32 stands for every block size from 32 tokens up (a power of two): a tile is then one 32-token part of a block
+    const int sub_mask = BS == 32 ? (a.sh.bs >> 5) - 1 : 0;
+    const int sub_shift = BS == 32 ? 31 - __builtin_clz(a.sh.bs >> 5) : 0;
+    const int bsz = BS == 32 ? a.sh.bs : BS;
     constexpr int ROWB = D * 2;            // bytes of a cache row
     constexpr int TILE = TOK * ROWB;       // bytes of one (block, head) of K or V
     constexpr int LROWV = ROWB + 32;       // LDS row stride of the V slot (the transposing reads are conflict free)
@@ -109,8 +113,9 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
         u4v v[VCH];
     };
     // the tile's two row groups: halves of the block `phys0`, or the 16-token blocks `phys0` and `phys1`
-    auto issue = [&](Block& blk, int phys0, int phys1) __attribute__((always_inline)) {
-        const long base0 = ((long)phys0 * Hkv + hkv) * (TILE / BPT);
+    auto issue = [&](Block& blk, int phys0, int phys1, int sub) __attribute__((always_inline)) {
+        const long base0 = BS == TOK ? ((long)phys0 * Hkv + hkv) * ((long)TILE * (a.sh.bs >> 5)) + (long)sub * TILE
+                                     : ((long)phys0 * Hkv + hkv) * (TILE / BPT);
         const long base1 = BS == TOK ? base0 + TILE / 2 : ((long)phys1 * Hkv + hkv) * (TILE / 2);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -124,11 +129,13 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
             blk.v[c] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(
                            a.value_cache + (c < VCH / 2 ? base0 : base1 - TILE / 2)) + c * 64 + lane);
     };
-    const int last_block = (kv_len + BS - 1) / BS - 1;  // a last tile of one 16-token block repeats it (rows masked)
+    const int last_block = (kv_len + bsz - 1) / bsz - 1;  // a last tile of one 16-token block repeats it (rows masked)
     Block ba, bb;
     int tile = tb + wv;
-    if (tile < te) issue(ba, table[min(BPT * tile, last_block)], table[min(BPT * tile + BPT - 1, last_block)]);
-    for (int i = tid; i < BPT * (te - tb); i += 64 * WAVES) tab[i] = table[min(BPT * tb + i, last_block)];
+    if (tile < te)
+        issue(ba, table[min((BPT * tile) >> sub_shift, last_block)], table[min((BPT * tile + BPT - 1) >> sub_shift, last_block)],
+              tile & sub_mask);
+    for (int i = tid; i < BPT * (te - tb); i += 64 * WAVES) tab[i] = table[min((BPT * tb + i) >> sub_shift, last_block)];
 
     // query operand (B of QK): lane (n, g) holds q[head n][32 s + 8 g + e]; heads beyond the group are zero
     s8v qreg[KS];
@@ -149,7 +156,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
 
     auto process = [&](Block& cur, Block& nxt, const int tl) __attribute__((always_inline)) {
         // next block's loads into flight, this block's V into the slot
-        if (tl + WAVES < te) issue(nxt, tab[BPT * (tl + WAVES - tb)], tab[BPT * (tl + WAVES - tb) + BPT - 1]);
+        if (tl + WAVES < te) issue(nxt, tab[BPT * (tl + WAVES - tb)], tab[BPT * (tl + WAVES - tb) + BPT - 1], (tl + WAVES) & sub_mask);
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
             const int piece = c * 64 + lane;
@@ -374,7 +381,7 @@ hipError_t launch_decode16_typed(hipStream_t s, const DecodeArgs& a, hipEvent_t 
 }  // namespace
 
 size_t decode16_table_bytes(int max_tiles, int block_size) {
-    return ((size_t)max_tiles * (TOK / block_size) * sizeof(int32_t) + 15) & ~(size_t)15;
+    return ((size_t)max_tiles * (block_size == 16 ? 2 : 1) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 
 // LDS in front of the block-table slice: V slots | per-wave (m, l) | [scores: block maxima | probabilities]
@@ -386,7 +393,7 @@ size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores) {
 
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,
                            hipEvent_t ev1) {
-    if ((a.sh.bs != 32 && a.sh.bs != 16) || a.G > 16 || (a.want_scores != 0) != (scores != nullptr)) return hipErrorInvalidValue;
+    if (a.sh.bs < 16 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1)) || a.G > 16 || (a.want_scores != 0) != (scores != nullptr)) return hipErrorInvalidValue;
     hipError_t e;
     if (a.sh.D == 128) e = dtype == DT_F16 ? launch_decode16_typed<128, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<128, DT_BF16>(s, a, ev0, ev1);
     else if (a.sh.D == 64) e = dtype == DT_F16 ? launch_decode16_typed<64, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<64, DT_BF16>(s, a, ev0, ev1);

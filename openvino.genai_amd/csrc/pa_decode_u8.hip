@@ -71,11 +71,12 @@ __device__ inline float xor_reduce_sum_g(float v) {
 // Loads one 32-token tile of K and V: whole-wave 16-byte passes plus the 16-chunk tails (K on lanes 0-15, V on 16-31).
 // With 32-token cache blocks the tile is the block `phys0`; with 16-token blocks its halves are the blocks `phys0` and
 // `phys1`, and each 16-byte chunk comes from the block its row lies in (the LDS image is the same).
+// `sub`: with cache blocks of 64 tokens or more, which 32-token part of the block `phys0` the tile is (0 otherwise).
 template <int FULL, int BS>
-__device__ __forceinline__ void issue_block(const DecodeArgs& a, int phys0, int phys1, int hkv, int tile_bytes, int lane,
+__device__ __forceinline__ void issue_block(const DecodeArgs& a, int phys0, int phys1, int sub, int hkv, int tile_bytes, int lane,
                                             u4v (&kraw)[FULL], u4v (&vraw)[FULL], u4v& traw) {
     if (BS == TOK) {
-        const long base = ((long)phys0 * a.sh.Hkv + hkv) * tile_bytes;
+        const long base = ((long)phys0 * a.sh.Hkv + hkv) * ((long)tile_bytes * (a.sh.bs >> 5)) + (long)sub * tile_bytes;
         const u4v* kp = reinterpret_cast<const u4v*>(a.key_cache + base);
         const u4v* vp = reinterpret_cast<const u4v*>(a.value_cache + base);
 #pragma unroll
@@ -105,6 +106,11 @@ template <int D, int QDT, int WAVES, int BS>
 __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs a) {
     constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile
     static_assert(BS == 32 || (BS == 16 && WAVES == 4), "the descriptor holds the ids of the first eight tiles");
+    // BS = 32 stands for every block size from 32 tokens up (a power of two): a tile is then one 32-token part of a
+    // block, the table slice in LDS holds the block id of every tile, and the part follows from the tile's number
+    const int sub_mask = BS == 32 ? (a.sh.bs >> 5) - 1 : 0;
+    const int sub_shift = BS == 32 ? 31 - __builtin_clz(a.sh.bs >> 5) : 0;
+    const int bsz = BS == 32 ? a.sh.bs : BS;
     constexpr int NT = 64 * WAVES;
     constexpr int ROW = D + 8;
     constexpr int TILE = TOK * ROW;        // bytes of one (block, head) of K or V
@@ -148,7 +154,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
     auto append_rows = [&]() __attribute__((always_inline)) {
         const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
-        const long dst = (((long)dsc->last_id * Hkv + hkv) * BS + (kv_len - 1) % BS) * ROW;
+        const long dst = (((long)dsc->last_id * Hkv + hkv) * bsz + (kv_len - 1) % bsz) * ROW;
         uint16_t kr[EPL], vr[EPL];
         load_row16<EPL>(a.key + src, kr);
         load_row16<EPL>(a.value + src, vr);
@@ -164,17 +170,17 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     u4v kraw[FULL], vraw[FULL], traw, kraw2[FULL], vraw2[FULL], traw2;
     int tile = tb + wv;
     if (tile < te)
-        issue_block<FULL, BS>(a, dsc->ids[BPT * wv], dsc->ids[BPT * wv + BPT - 1], hkv, TILE, lane, kraw, vraw, traw);
+        issue_block<FULL, BS>(a, dsc->ids[BPT * wv], dsc->ids[BPT * wv + BPT - 1], tile & sub_mask, hkv, TILE, lane, kraw, vraw, traw);
     if (tile + WAVES < te)
-        issue_block<FULL, BS>(a, dsc->ids[BPT * (wv + WAVES)], dsc->ids[BPT * (wv + WAVES) + BPT - 1], hkv, TILE, lane, kraw2,
-                              vraw2, traw2);
+        issue_block<FULL, BS>(a, dsc->ids[BPT * (wv + WAVES)], dsc->ids[BPT * (wv + WAVES) + BPT - 1], (tile + WAVES) & sub_mask,
+                              hkv, TILE, lane, kraw2, vraw2, traw2);
     if (appends && !append_first) append_rows();
     // this workgroup's slice of the block table, so that no later block fetch waits on a table fetch
     int32_t* tab = reinterpret_cast<int32_t*>(smem + a.table_off);
     // (16-token blocks: two ids per tile; a last tile of one block repeats it, its second half lies beyond kv_len)
     {
-        const int last_block = (kv_len + BS - 1) / BS - 1;
-        for (int i = tid; i < BPT * (te - tb); i += NT) tab[i] = table[min(BPT * tb + i, last_block)];
+        const int last_block = (kv_len + bsz - 1) / bsz - 1;
+        for (int i = tid; i < BPT * (te - tb); i += NT) tab[i] = table[min((BPT * tb + i) >> sub_shift, last_block)];
     }
 
     // query operand (B of QK): lane (n, g) holds q[head n][32 s + 8 g + e]
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
         if (lane >= 16 && lane < 32) reinterpret_cast<u4v*>(slot)[FULL * 64 + lane - 16] = tr;
         if (tile + 2 * WAVES < te) {
             const int ti = BPT * (tile + 2 * WAVES - tb);
-            issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], hkv, TILE, lane, kr, vr, tr);
+            issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], (tile + 2 * WAVES) & sub_mask, hkv, TILE, lane, kr, vr, tr);
         }
         __builtin_amdgcn_wave_barrier();
 
@@ -661,7 +667,7 @@ size_t decode_u8_lds_bytes(int D, int G, int max_tiles, bool want_scores, int wa
     if (want_scores) bytes += (size_t)max_tiles * 16 * sizeof(float) + (size_t)G * max_tiles * TOK * sizeof(uint16_t);
     bytes = (bytes + 15) & ~(size_t)15;
     *table_off = (int32_t)bytes;
-    bytes += (size_t)max_tiles * (TOK / block_size) * sizeof(int32_t);
+    bytes += (size_t)max_tiles * (block_size == 16 ? 2 : 1) * sizeof(int32_t);
     return (bytes + 15) & ~(size_t)15;
 }
 
@@ -687,7 +693,7 @@ static hipError_t launch_decode_waves(hipStream_t s, const DecodeArgs& a, float*
         if (a.waves != 4) return hipErrorInvalidValue;
         return launch_decode_typed<D, QDT, 4, 16>(s, a, scores, max_kv_len, ev0, ev1);
     }
-    if (a.sh.bs != 32) return hipErrorInvalidValue;
+    if (a.sh.bs < 32 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1))) return hipErrorInvalidValue;
     if (a.waves == 8) return launch_decode_typed<D, QDT, 8, 32>(s, a, scores, max_kv_len, ev0, ev1);
     return launch_decode_typed<D, QDT, 4, 32>(s, a, scores, max_kv_len, ev0, ev1);
 }

@@ -244,7 +244,9 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
             const int32_t per = (hi - lo + nsplit - 1) / nsplit;
             const int32_t* tab = ids + ctx->h_bib[b];
             // cache blocks per 32-token tile, and the sequence's last block (a last tile of one 16-token block repeats it)
-            const int32_t bpt = 32 / ctx->cfg.block_size, last_block = (kv_len - 1) / ctx->cfg.block_size;
+            // (blocks of 64 tokens or more: one id per tile, that of the block the tile is a part of)
+            const int32_t bs = ctx->cfg.block_size, bpt = bs == 16 ? 2 : 1, last_block = (kv_len - 1) / bs;
+            const int32_t sub_shift = bs <= 32 ? 0 : __builtin_ctz((unsigned)(bs / 32));
             for (int32_t s = 0; s < nsplit; ++s) {
                 pa::DecodeDesc& d = out[i * nsplit + s];
                 d.b = b;
@@ -257,7 +259,7 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
                 d.score_off = soff[b];
                 d.last_id = tab[last_block];
                 for (int32_t j = 0; j < 16; ++j)
-                    d.ids[j] = bpt * d.tb + j < bpt * d.te ? tab[std::min(bpt * d.tb + j, last_block)] : 0;
+                    d.ids[j] = bpt * d.tb + j < bpt * d.te ? tab[std::min((bpt * d.tb + j) >> sub_shift, last_block)] : 0;
             }
         }
     }
@@ -270,23 +272,26 @@ void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
                                    ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
 }
 
-// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).  The tuned kernels'
-// tiles are 32 tokens: one 32-token cache block or two 16-token ones.
+// Block sizes the tuned kernels take.  Their tiles are 32 tokens: two 16-token cache blocks, one 32-token block, or a
+// 32-token part of a block of 64, 128 or 256 tokens.
+bool tuned_block_size(int32_t bs) { return bs >= 16 && bs <= 256 && (bs & (bs - 1)) == 0; }
+
+// Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).
 bool decode_u8_shape(const pa_config& c) {
-    return c.kv_cache_dtype == PA_U8 && (c.block_size == 32 || c.block_size == 16) &&
+    return c.kv_cache_dtype == PA_U8 && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
 bool mfma_shape(const pa_config& c) {
-    return (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && (c.block_size == 32 || c.block_size == 16) &&
+    return (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 256;
 }
 
 // Shapes the 16-bit decode kernel is built for (single-token sequences of a call that asks for no scores).
 bool decode16_shape(const pa_config& c) {
-    return c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && (c.block_size == 32 || c.block_size == 16) &&
+    return c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
@@ -339,7 +344,7 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
     // A context whose probabilities do not fit half a CU's LDS is cut into splits that send every head's
     // probabilities through HBM and add a merge.  With enough (sequence, kv head) pairs to give every CU a workgroup
     // of its own, one workgroup of eight waves per CU (the same waves per CU, the whole LDS) needs fewer of them.
-    if (u8 && c.block_size == 32 && most > cap4 && pairs >= 256) {
+    if (u8 && c.block_size >= 32 && most > cap4 && pairs >= 256) {
         int32_t cap8 = 0;
         const int32_t s8 = plan(8, 256, &cap8);
         if (s8 < s) {
@@ -1008,8 +1013,9 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
             if (had) plan_items(ctx);
             return;
         }
-        PA_REQUIRE(mfma_shape(c) && c.block_size == 32, PA_NOT_IMPLEMENTED,
-                   "block-sparse prefill needs block_size 32, head_size 64 or 128 and a u8 cache or one of the query's type");
+        PA_REQUIRE(mfma_shape(c) && c.block_size >= 32, PA_NOT_IMPLEMENTED,
+                   "block-sparse prefill needs a block_size of 32 to 256 (a power of two), head_size 64 or 128 and a u8 cache "
+                   "or one of the query's type");
         auto pow2 = [](int32_t v) { return v > 0 && (v & (v - 1)) == 0; };
         PA_REQUIRE(pow2(block_size) && block_size >= 32, PA_NOT_IMPLEMENTED,
                    "xattention_block_size must be a power of two, at least 32");

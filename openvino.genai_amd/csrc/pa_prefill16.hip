@@ -329,9 +329,11 @@ void pa_prefill16_kernel(PrefillArgs a) {
     // fetched from the block it lies in (a last tile of one block repeats it; those rows lie beyond kv_len).
     // tile_base(tile, upper): what to add to `row * CROWB` for a row of the tile's lower or upper half.
     const bool bs16 = a.sh.bs == 16;
+    const int sub_mask = bs16 ? 0 : (a.sh.bs >> 5) - 1, sub_shift = bs16 ? 0 : 31 - __builtin_clz(a.sh.bs >> 5);
     const int last_block16 = (kv_len - 1) >> 4;
     auto tile_base = [&](int tile, bool upper) __attribute__((always_inline)) -> long {
-        if (!bs16) return ((long)table[tile] * Hkv + hkv) * (TOK * CROWB);
+        // (blocks of 32 tokens or more, a power of two: the tile is one 32-token part of its block)
+        if (!bs16) return ((long)table[tile >> sub_shift] * Hkv + hkv) * ((long)a.sh.bs * CROWB) + (long)(tile & sub_mask) * (TOK * CROWB);
         const long lo = ((long)table[2 * tile] * Hkv + hkv) * (16 * CROWB);
         const long hi = ((long)table[min(2 * tile + 1, last_block16)] * Hkv + hkv) * (16 * CROWB) - 16 * CROWB;
         return upper ? hi : lo;

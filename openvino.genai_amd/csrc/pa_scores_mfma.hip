@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
     if (base >= kv_len) return;
     const int W = st.score_window[b];
     const int Hq = sh.Hq, Hkv = sh.Hkv, G = Hq / Hkv;
-    const int bs_shift = sh.bs == 16 ? 4 : 5;  // cache blocks of 16 or 32 tokens
+    const int bs_shift = 31 - __builtin_clz(sh.bs);  // cache blocks of 16 to 256 tokens (a power of two)
     const int R = W * G;                       // query rows per kv head
     const int first_tok = t0 + q_len - W;      // first of the last W tokens
     const int first_pos = past + q_len - W;    // its position
@@ -219,7 +219,7 @@ hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& s
                            block_indices, final_ml, scores, seq_list, n_seqs, xd, ss);                         \
         return hipGetLastError();                                                                              \
     }
-    if (sh.bs != 32 && sh.bs != 16) return hipErrorInvalidValue;
+    if (sh.bs < 16 || sh.bs > 256 || (sh.bs & (sh.bs - 1))) return hipErrorInvalidValue;
     if (kv_dtype == DT_U8) {
         if (sh.D == 64 && q_dtype == DT_F16) PA_REPLAY(64, DT_F16, DT_F16, true)
         if (sh.D == 64 && q_dtype == DT_BF16) PA_REPLAY(64, DT_F16, DT_BF16, true)

@@ -81,6 +81,7 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
     const int kv_len = past + q_len;
     const int S = 1 << a.s_shift;
     const int32_t* table = a.block_indices + a.st.block_indices_begins[b];
+    const int bs_shift = 31 - __builtin_clz(a.sh.bs);  // cache blocks of 32 tokens or more (a power of two)
 
     // this thread's share of a stage's key rows: rows kr0 + RPP * k, the piece `kpart` of each
     const int kr0 = U8 ? tid >> 2 : tid >> 3, kpart = U8 ? tid & 3 : tid & 7;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
     for (int k = 0; k < KCH; ++k) {
         k_pos0[k] = (KT * tl.jc + kr0 + RPP * k) << a.s_shift;
         const int pos = min(k_pos0[k], kv_len - 1);
-        k_blk[k] = a.key_cache + ((long)table[pos >> 5] * Hkv + hkv) * (32 * CROWB);
+        k_blk[k] = a.key_cache + ((long)table[pos >> bs_shift] * Hkv + hkv) * ((long)a.sh.bs * CROWB);
     }
     // this wave's query rows: position of slot 0 (the group's last token), relative to the chunk
     int q_rel0[2];
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
         const int s = u / DP, ch = (u % DP) * 64;
 #pragma unroll
         for (int k = 0; k < KCH; ++k) {
-            const uint8_t* row = k_blk[k] + (min(k_pos0[k] + s, kv_len - 1) & 31) * CROWB;
+            const uint8_t* row = k_blk[k] + (min(k_pos0[k] + s, kv_len - 1) & (a.sh.bs - 1)) * CROWB;
             if (U8) {
                 ks.c[k] = *reinterpret_cast<const u4v*>(row + 8 + ch + 16 * kpart);
                 ks.hd[k] = *reinterpret_cast<const uint2*>(row);
@@ -409,7 +410,7 @@ hipError_t launch_xattention(hipStream_t s, const XattArgs& a, int q_dtype, int 
 #define PA_XLOGITS(DD, DT, Q, U8) \
     hipLaunchKernelGGL((xatt_logits_kernel<DD, DT, Q, U8>), lgrid, dim3(256), 0, s, a)
     const bool f16q = q_dtype == DT_F16;
-    if (a.sh.bs != 32 || (a.sh.D != 64 && a.sh.D != 128)) return hipErrorInvalidValue;
+    if (a.sh.bs < 32 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1)) || (a.sh.D != 64 && a.sh.D != 128)) return hipErrorInvalidValue;
     if (kv_dtype == DT_U8) {
         if (a.sh.D == 64) { if (f16q) PA_XLOGITS(64, DT_F16, DT_F16, true); else PA_XLOGITS(64, DT_F16, DT_BF16, true); }
         else { if (f16q) PA_XLOGITS(128, DT_F16, DT_F16, true); else PA_XLOGITS(128, DT_F16, DT_BF16, true); }

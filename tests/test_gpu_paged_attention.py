@@ -263,14 +263,28 @@ BLOCK16 = [
     ("b16_u8_bf16q_d64_g8", (16, 2, 64, 16, "bf16", "u8", [0, 31, 16, 500], [33, 100, 1, 17]), {}),
     ("b16_u8_window", (8, 2, 128, 16, "f16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
     ("b16_u8_odd_block_counts", (8, 2, 128, 16, "f16", "u8", [0, 3, 20], [17, 45, 60]), {}),
+    # blocks of 64, 128 and 256 tokens (256 is what the reference's GPU plugin uses with XAttention): a tile is a
+    # 32-token part of a block
+    ("b64_u8_decode", (8, 2, 128, 64, "f16", "u8", [0, 31, 32, 63, 64, 65, 700, 3000], [1] * 8), {}),
+    ("b256_u8_decode_multi_split", (32, 8, 128, 256, "f16", "u8", [9000, 4100, 255, 256, 257, 33], [1] * 6), {}),
+    ("b128_u8_decode_window", (8, 2, 64, 128, "bf16", "u8", [5000, 900, 40, 300], [1] * 4), {"sliding_window": 1000}),
+    ("b256_bf16_decode", (28, 4, 128, 256, "bf16", "bf16", [1000, 2047, 5, 255, 256], [1] * 5), {}),
+    ("b64_f16_decode_long", (8, 2, 128, 64, "f16", "f16", [15000, 63], [1, 1]), {}),
+    ("b256_bf16_g7_mixed", (28, 4, 128, 256, "bf16", "bf16", [0, 700, 333, 40, 2000], [150, 37, 1, 1, 64]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3]}),
+    ("b128_f16_chunks_only_window", (4, 4, 128, 128, "f16", "f16", [300, 0], [200, 130]), {"sliding_window": 100}),
+    ("b256_u8_g4_mixed", (32, 8, 128, 256, "f16", "u8", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
+    ("b64_u8_bf16q_d64_g8", (16, 2, 64, 64, "bf16", "u8", [0, 31, 64, 500], [33, 100, 1, 17]), {}),
+    ("b256_bf16_long_singles", (8, 2, 128, 256, "bf16", "bf16", [0, 5000, 2049], [50, 1, 1]), {}),
 ]
 
 
 @pytest.mark.parametrize("name,args,kw", BLOCK16, ids=[c[0] for c in BLOCK16])
 def test_block_size_16_steps(pkg, dev, name, args, kw):
-    """Caches of 16-token blocks (the block size of the reference's GPU plugin) on the tuned kernels, whose 32-token
-    tiles are then two blocks: single-token steps, chunks and mixed steps, with and without scores, appended rows
-    included."""
+    """Caches of 16-token blocks (the block size of the reference's GPU plugin) and of 64 to 256 tokens on the tuned
+    kernels, whose 32-token tiles are then two blocks, or a part of one: single-token steps, chunks and mixed steps, with
+    and without scores, appended rows included."""
     got, ref, c = _check(pkg, dev, H.case_from_lens(name, *args, **kw), 59, outliers=True)
     got2 = H.run_case_on_gpu(pkg, c, dev, want_scores=False)
     H.assert_close(got2["out"], ref["out"], c["q_dtype"])

@@ -137,6 +137,19 @@ def test_mixed_step(env):
         _check(pkg, dev, c, np.array([0.8, 0.8, 0.0, 0.0, 0.7], np.float32), 64, 8)
 
 
+def test_mixed_step_with_256_token_cache_blocks(env):
+    """The block size the reference's GPU plugin uses with XAttention: 256-token cache blocks, key blocks of 256 and of
+    64 positions."""
+    pkg, dev = env
+    past = [300, 40, 2000, 511, 900]
+    new = [200, 1, 130, 1, 64]
+    for kd, xb, bs in (("u8", 256, 256), ("bf16", 64, 256), ("bf16", 128, 64)):
+        case = H.case_from_lens("mixed_b256", 16, 4, 128, bs, "bf16", kd, past, new, scale=4.0 / np.sqrt(128),
+                                score_aggregation_window=[4, 1, 0, 1, 64])
+        c = H.build_case(case, 98, outliers=True)
+        _check(pkg, dev, c, np.array([0.8, 0.8, 0.0, 0.0, 0.7], np.float32), xb, 8)
+
+
 def test_threshold_zero_is_dense(env):
     pkg, dev = env
     case = H.case_from_lens("dense", 8, 2, 128, 32, "f16", "u8", [100, 30], [200, 1])

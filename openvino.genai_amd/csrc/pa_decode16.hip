@@ -102,8 +102,8 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
 
     uint8_t* slot = smem + wv * SLOT;                                  // this wave's V block
     float* wave_ml = reinterpret_cast<float*>(smem + WAVES * SLOT);    // [WAVES][16][2]
-    float* msnap = wave_ml + WAVES * 16 * 2;                           // [max_tiles][16] running maximum at each block
-    _Float16* ptile = reinterpret_cast<_Float16*>(msnap + (a.want_scores ? a.max_tiles * 16 : 0));  // [G][max_tiles * TOK]
+    float* msnap = wave_ml + WAVES * 16 * 2;                           // [max_tiles][G] running maximum at each block
+    _Float16* ptile = reinterpret_cast<_Float16*>(msnap + (a.want_scores ? decode16_snap_floats(a.max_tiles, G) : 0));  // [G][max_tiles * TOK]
     const int pstride = a.max_tiles * TOK;
     int32_t* tab = reinterpret_cast<int32_t*>(smem + a.table_off);     // the workgroup's slice of the block table
 
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
                 _Float16* dst = ptile + n * pstride + lt * TOK + 4 * g;
                 *reinterpret_cast<h4*>(dst) = h4{(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3]};
                 *reinterpret_cast<h4*>(dst + 16) = h4{(_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
-                if (g == 0) msnap[lt * 16 + n] = m_safe;
+                if (g == 0) msnap[lt * G + n] = m_safe;
             }
         }
         __builtin_amdgcn_wave_barrier();  // the slot was written by this wave's own lanes
@@ -270,11 +270,25 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
     const float inv_l = L > 0.0f ? 1.0f / L : 0.0f;
     if (a.want_scores) {
         // one factor per (block, head): exp2(snapshot - M) (/ L when this workgroup saw the whole context), written
-        // over the snapshot.  Entry e belongs to head e % 16 = this thread's n; the barrier inside the merge below
-        // publishes the factors
-        const float fl = final_out ? inv_l : 1.0f;
-        for (int e = tid; e < max(te - tb, 0) * 16; e += 64 * WAVES)
-            msnap[e] = n < G ? __builtin_amdgcn_exp2f(msnap[e] - M) * fl : 0.0f;
+        // over the snapshot; entry e belongs to head e % G, whose M and L are folded again from the waves' values
+        // (in the order used above).  The barrier inside the merge below publishes the factors
+        for (int e = tid; e < max(te - tb, 0) * G; e += 64 * WAVES) {
+            const int h = e % G;
+            float Mh = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) Mh = fmaxf(Mh, wave_ml[(w * 16 + h) * 2]);
+            float fl = 1.0f;
+            if (final_out) {
+                float Lh = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) {
+                    const float mw = wave_ml[(w * 16 + h) * 2];
+                    Lh += (mw == -INFINITY) ? 0.0f : wave_ml[(w * 16 + h) * 2 + 1] * __builtin_amdgcn_exp2f(mw - Mh);
+                }
+                fl = Lh > 0.0f ? 1.0f / Lh : 0.0f;
+            }
+            msnap[e] = __builtin_amdgcn_exp2f(msnap[e] - Mh) * fl;
+        }
     }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
@@ -324,7 +338,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
         for (int pos = tid; pos < p0; pos += 64 * WAVES) dst[pos] = 0.0f;
         const int cnt = kv_len - p0;
         for (int lp = 4 * tid; lp < cnt; lp += 4 * 64 * WAVES) {
-            const float* f = fac + (lp / TOK) * 16;
+            const float* f = fac + (lp / TOK) * G;
             f4 sum = f4{0.0f, 0.0f, 0.0f, 0.0f};
             for (int h = 0; h < G; ++h) {
                 const h4 p4 = *reinterpret_cast<const h4*>(ptile + h * pstride + lp);
@@ -349,7 +363,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
             _Float16* dst = a.p_split + (long)(hkv * G + h) * stride + aoff;
             for (int pos = p_lo + 4 * tid; pos < p_hi; pos += 4 * 64 * WAVES) {
                 const int lp = pos - p_lo;
-                const float fh = fac[(lp / TOK) * 16 + h];
+                const float fh = fac[(lp / TOK) * G + h];
                 const h4 p4 = *reinterpret_cast<const h4*>(ptile + h * pstride + lp);
                 *reinterpret_cast<h4*>(dst + pos) = h4{(_Float16)((float)p4[0] * fh), (_Float16)((float)p4[1] * fh),
                                                        (_Float16)((float)p4[2] * fh), (_Float16)((float)p4[3] * fh)};
@@ -387,7 +401,7 @@ size_t decode16_table_bytes(int max_tiles, int block_size) {
 // LDS in front of the block-table slice: V slots | per-wave (m, l) | [scores: block maxima | probabilities]
 size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores) {
     size_t bytes = (size_t)4 * TOK * (D * 2 + 32) + 4 * 16 * 2 * sizeof(float);
-    if (want_scores) bytes += (size_t)max_tiles * 16 * sizeof(float) + (size_t)G * max_tiles * TOK * sizeof(uint16_t);
+    if (want_scores) bytes += (size_t)decode16_snap_floats(max_tiles, G) * sizeof(float) + (size_t)G * max_tiles * TOK * sizeof(uint16_t);
     return (bytes + 15) & ~(size_t)15;
 }
 

@@ -227,6 +227,8 @@ struct XattDev {            // what the attention and score kernels need of it (
 
 // The 16-bit-cache decode kernel (pa_decode16.hip): takes the arguments of the u8 family and leaves split partials,
 // per-kv-head score sums and split probabilities in its layouts (table_off is set by the launcher).
+// floats of the 16-bit decode kernel's per-(block, head) maxima in LDS (the probabilities behind them stay 16-byte aligned)
+__host__ __device__ inline int decode16_snap_floats(int max_tiles, int G) { return (max_tiles * G + 3) & ~3; }
 size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores);
 size_t decode16_table_bytes(int max_tiles, int block_size);  // the block-table slice behind it
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,

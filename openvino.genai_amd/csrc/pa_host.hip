@@ -317,11 +317,12 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
                       : pa::decode16_lds_bytes(c.head_size, G, tiles, want_scores) + pa::decode16_table_bytes(tiles, c.block_size);
         };
         // the score path keeps a split's probabilities in LDS: that bounds the blocks per workgroup
-        const size_t budget = (size_t)(160 * 1024 / (slots / 256)) - 1280;
+        const size_t budget = (size_t)(160 * 1024 / (slots / 256));
+        auto fits = [&](int32_t tiles) { return (lds_of(tiles) + 1279) / 1280 * 1280 <= budget; };
         int32_t cap = most;
         if (want_scores) {
-            cap = std::min<int32_t>(most, (int32_t)(budget / (64 + 64 * G + 4)));
-            while (cap > 1 && lds_of(cap) > budget) --cap;
+            cap = std::min<int32_t>(most, (int32_t)(budget / (64 * G)));
+            while (cap > 1 && !fits(cap)) --cap;
         }
         int32_t s = 1;
         // aim for at least one round of workgroups, keep at least 16 blocks per workgroup (with fewer, what the

@@ -219,6 +219,9 @@ DECODE16 = [
     ("bf16_long_splits_window", (16, 8, 128, 32, "bf16", "bf16", [9000, 4000], [1, 1]), {"sliding_window": 2500}),
     ("f16_window_inside_block", (8, 2, 128, 32, "f16", "f16", [100, 45, 700], [1] * 3), {"sliding_window": 40}),
     ("bf16_mixed_with_chunks", (8, 2, 128, 32, "bf16", "bf16", [500, 0, 2000, 64], [1, 70, 1, 300]), {}),
+    # odd products of blocks x heads: the per-block maxima in LDS are packed G to a block
+    ("bf16_d128_g5_odd_blocks", (10, 2, 128, 32, "bf16", "bf16", [4127, 95, 33], [1] * 3), {}),
+    ("f16_d128_g5_long_splits", (5, 1, 128, 32, "f16", "f16", [12001], [1]), {}),
     ("f16_g17_stays_on_the_matrix_kernel", (17, 1, 64, 32, "f16", "f16", [200, 77], [1, 1]), {}),
 ]
 

@@ -58,21 +58,30 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     constexpr int CROWB = U8 ? D + 8 : D * 2;
     constexpr int DP = D / 64;             // stages per slot
-    constexpr int KST = 128 + 16;          // LDS bytes per key row of a stage (padded: the operand reads are conflict free)
+    constexpr int KST = 128;               // LDS bytes per key or query row of a stage; the row's 16-byte piece p sits at
+                                           // p ^ ((row >> 1) & 7): stores (eight or four lanes to a row) and operand
+                                           // reads (sixteen rows at one piece) both touch every bank once
     constexpr int KT = XATT_KEY_TILE;      // strided key groups per workgroup
     constexpr int NJ = KT / 16;
     constexpr int RPP = U8 ? 64 : 32;      // key rows one pass of the 256 threads covers
     constexpr int KCH = KT / RPP;          // 16-byte pieces of the cache a thread moves per stage
     __shared__ __align__(16) uint8_t kbuf[2][KT * KST];
+    __shared__ __align__(16) uint8_t qbuf[2][4][32 * KST];   // per wave: its head's 32 query rows of a stage
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int Hq = a.sh.Hq, Hkv = a.sh.Hkv, G = a.G;
     const int nsub = (G + 3) >> 2;
-    const int hkv = blockIdx.y / nsub;
-    const int hg = (blockIdx.y % nsub) * 4 + wv;   // head within the group; waves beyond it repeat the last head
+    // Workgroup i runs on XCD i % 8, each with an L2 of its own.  The work is numbered (kv head, tile, set of four
+    // heads) -- tiles in the order (sequence, query tile, key tile) -- and each XCD takes a contiguous eighth of that
+    // numbering, so that the workgroups that read the same query rows (all key tiles of a query tile) and the same key
+    // rows (both query tiles, all head sets) meet in one L2 instead of each fetching them over the fabric.
+    const int total = gridDim.x, xcd = blockIdx.x & 7;
+    const int work = xcd * (total >> 3) + min(xcd, total & 7) + (blockIdx.x >> 3);
+    const int hkv = work / (a.ntiles * nsub);
+    const int hg = (work % nsub) * 4 + wv;          // head within the group; waves beyond it repeat the last head
     const bool head_ok = hg < G;
     const int hq = hkv * G + min(hg, G - 1);
-    const XattTile tl = a.tiles[blockIdx.x];
+    const XattTile tl = a.tiles[(work / nsub) % a.ntiles];
     const XattSeq xs = a.seqs[tl.x];
     const int b = xs.b;
     const int t0 = a.st.subsequence_begins[b];
@@ -93,13 +102,12 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
         const int pos = min(k_pos0[k], kv_len - 1);
         k_blk[k] = a.key_cache + ((long)table[pos >> bs_shift] * Hkv + hkv) * ((long)a.sh.bs * CROWB);
     }
-    // this wave's query rows: position of slot 0 (the group's last token), relative to the chunk
-    int q_rel0[2];
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi) q_rel0[mi] = ((xs.qs0 + 32 * tl.it + 16 * mi + n) << a.s_shift) + S - 1 - past;
-
+    // this wave's query rows: a load covers eight rows, eight lanes to a row's 128 bytes; position of slot 0 (the
+    // group's last token) of this lane's row in the first load, relative to the chunk
+    const int qrow = lane >> 3, qpart = lane & 7;
+    const int q_rel0 = ((xs.qs0 + 32 * tl.it + qrow) << a.s_shift) + S - 1 - past;
     struct KSet { u4v c[KCH]; uint2 hd[KCH]; };   // hd: u8 row headers
-    struct QSet { u4v q[2][2]; };
+    struct QSet { u4v q[4]; };
     auto load_k = [&](KSet& ks, int u) __attribute__((always_inline)) {
         const int s = u / DP, ch = (u % DP) * 64;
 #pragma unroll
@@ -119,7 +127,8 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
 #pragma unroll
         for (int k = 0; k < KCH; ++k) {
             const bool ok = k_pos0[k] + s < kv_len;
-            uint8_t* dst = buf + (kr0 + RPP * k) * KST + (U8 ? 32 : 16) * kpart;
+            const int krow = kr0 + RPP * k, ksw = (krow >> 1) & 7;
+            uint8_t* dst = buf + krow * KST;
             if (U8) {
                 const float sc = ok ? __builtin_bit_cast(float, ks.hd[k].x) : 0.0f;
                 const float nz = ok ? -__builtin_bit_cast(float, ks.hd[k].y) * sc : 0.0f;
@@ -130,21 +139,36 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
                     v[e >> 1][2 * (e & 1)] = f16x2(fmaf((float)(w & 0xffu), sc, nz), fmaf((float)((w >> 8) & 0xffu), sc, nz));
                     v[e >> 1][2 * (e & 1) + 1] = f16x2(fmaf((float)((w >> 16) & 0xffu), sc, nz), fmaf((float)(w >> 24), sc, nz));
                 }
-                *reinterpret_cast<u4v*>(dst) = v[0];
-                *reinterpret_cast<u4v*>(dst + 16) = v[1];
+                *reinterpret_cast<u4v*>(dst + 16 * ((2 * kpart) ^ ksw)) = v[0];
+                *reinterpret_cast<u4v*>(dst + 16 * ((2 * kpart + 1) ^ ksw)) = v[1];
             } else {
-                *reinterpret_cast<u4v*>(dst) = ok ? ks.c[k] : u4v{0u, 0u, 0u, 0u};
+                *reinterpret_cast<u4v*>(dst + 16 * (kpart ^ ksw)) = ok ? ks.c[k] : u4v{0u, 0u, 0u, 0u};
             }
         }
     };
     auto load_q = [&](QSet& qs, int u) __attribute__((always_inline)) {
-        const int s = u / DP, ch = (u % DP) * 64 + 16 * g;
+        const int s = u / DP, ch = (u % DP) * 64 + 8 * qpart;
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
-            const int rel = q_rel0[mi] - s;
-            const uint16_t* p = a.query + ((long)(t0 + min(max(rel, 0), q_len - 1)) * Hq + hq) * D + ch;
-            qs.q[mi][0] = *reinterpret_cast<const u4v*>(p);
-            qs.q[mi][1] = *reinterpret_cast<const u4v*>(p + 8);
+        for (int c = 0; c < 4; ++c) {
+            const int rel = q_rel0 + ((8 * c) << a.s_shift) - s;
+            qs.q[c] = *reinterpret_cast<const u4v*>(a.query + ((long)(t0 + min(max(rel, 0), q_len - 1)) * Hq + hq) * D + ch);
+        }
+    };
+    // rows outside the chunk go in as zeros; a bf16 query against f16 operands is converted here
+    auto store_q = [&](const QSet& qs, int u) __attribute__((always_inline)) {
+        const int s = u / DP;
+        uint8_t* buf = qbuf[u & 1][wv];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int rel = q_rel0 + ((8 * c) << a.s_shift) - s;
+            u4v v = (rel >= 0 && rel < q_len) ? qs.q[c] : u4v{0u, 0u, 0u, 0u};
+            if (QDT != DT) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] = f16x2(__builtin_bit_cast(float, v[e] << 16), __builtin_bit_cast(float, v[e] & 0xffff0000u));
+            }
+            const int row = 8 * c + qrow;
+            *reinterpret_cast<u4v*>(buf + row * KST + 16 * (qpart ^ ((row >> 1) & 7))) = v;
         }
     };
     f4 acc[2][NJ];
@@ -152,53 +176,52 @@ __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int nj = 0; nj < NJ; ++nj) acc[mi][nj] = f4{0.0f, 0.0f, 0.0f, 0.0f};
-    auto compute = [&](const QSet& qs, int u) __attribute__((always_inline)) {
-        const int s = u / DP;
+    auto compute = [&](int u) __attribute__((always_inline)) {
         const uint8_t* buf = kbuf[u & 1];
-        s8v qop[2][2];
+        const uint8_t* qb = qbuf[u & 1][wv];
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
-            const int rel = q_rel0[mi] - s;
-            const bool ok = rel >= 0 && rel < q_len;
+        for (int kk = 0; kk < 2; ++kk) {
+            s8v qop[2];
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                u4v v = ok ? qs.q[mi][kk] : u4v{0u, 0u, 0u, 0u};
-                if (QDT != DT) {  // bf16 query against f16 operands
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        v[e] = f16x2(__builtin_bit_cast(float, v[e] << 16), __builtin_bit_cast(float, v[e] & 0xffff0000u));
-                }
-                qop[mi][kk] = __builtin_bit_cast(s8v, v);
-            }
-        }
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+            for (int mi = 0; mi < 2; ++mi)
+                qop[mi] = *reinterpret_cast<const s8v*>(qb + (16 * mi + n) * KST + 16 * ((2 * g + kk) ^ ((n >> 1) & 7)));
 #pragma unroll
             for (int nj = 0; nj < NJ; ++nj) {
-                const s8v kop = *reinterpret_cast<const s8v*>(buf + (16 * nj + n) * KST + 32 * g + 16 * kk);
+                const s8v kop = *reinterpret_cast<const s8v*>(buf + (16 * nj + n) * KST + 16 * ((2 * g + kk) ^ ((n >> 1) & 7)));
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi) acc[mi][nj] = mma<DT>(kop, qop[mi][kk], acc[mi][nj]);
+                for (int mi = 0; mi < 2; ++mi) acc[mi][nj] = mma<DT>(kop, qop[mi], acc[mi][nj]);
             }
+        }
     };
 
-    // stage u: its key rows were asked for in iteration u - 2 and written to LDS in iteration u - 1, its query rows
-    // asked for in iteration u - 1; the workgroups sharing a CU cover for each other
+    // stage u: its key and query rows were asked for in iteration u - 2 and written to LDS in iteration u - 1 (the
+    // buffers (u + 1) & 1 were last read in iteration u - 1); the workgroups sharing a CU cover for each other.
+    // (Four stages of loads in flight instead of one changed nothing: the pace is set by bytes, not by latency.)
     const int NU = S * DP;
     KSet k0, k1;
     QSet q0, q1;
     load_k(k0, 0);
     load_q(q0, 0);
-    if (NU > 1) load_k(k1, 1);
+    if (NU > 1) {
+        load_k(k1, 1);
+        load_q(q1, 1);
+    }
     store_k(k0, 0);
+    store_q(q0, 0);
     __syncthreads();
 #define PA_XSTEP(KA, KB, QA, QB, U)                                      \
     {                                                                    \
         const int u = (U);                                               \
         if (u >= NU) break;                                              \
-        if (u + 1 < NU) store_k(KB, u + 1);  /* buffer (u + 1) & 1 was last read in iteration u - 1 */ \
-        if (u + 2 < NU) load_k(KA, u + 2);   /* set of stage u: it went to LDS in iteration u - 1 */ \
-        if (u + 1 < NU) load_q(QB, u + 1);   /* set of stage u - 1 */   \
-        compute(QA, u);                                                  \
+        if (u + 1 < NU) {                                                \
+            store_k(KB, u + 1);                                          \
+            store_q(QB, u + 1);                                          \
+        }                                                                \
+        if (u + 2 < NU) {                                                \
+            load_k(KA, u + 2);                                           \
+            load_q(QA, u + 2);                                           \
+        }                                                                \
+        compute(u);                                                      \
         __syncthreads();                                                 \
     }
     for (int i = 0;; i += 2) {
@@ -406,7 +429,7 @@ __global__ __launch_bounds__(64) void xatt_item_keep_kernel(XattArgs a) {
 
 hipError_t launch_xattention(hipStream_t s, const XattArgs& a, int q_dtype, int kv_dtype) {
     if (a.nseq == 0) return hipSuccess;
-    const dim3 lgrid((unsigned)a.ntiles, (unsigned)(a.sh.Hkv * ceil_div(a.G, 4)));
+    const dim3 lgrid((unsigned)(a.ntiles * a.sh.Hkv * ceil_div(a.G, 4)));
 #define PA_XLOGITS(DD, DT, Q, U8) \
     hipLaunchKernelGGL((xatt_logits_kernel<DD, DT, Q, U8>), lgrid, dim3(256), 0, s, a)
     const bool f16q = q_dtype == DT_F16;

@@ -50,9 +50,11 @@ __device__ __forceinline__ uint32_t f16x2(float a, float b) {
 // channels).  The stage's key rows (128 bytes each as 16-bit values) go global -> registers -> LDS once per
 // workgroup and serve all four heads -- read straight from global memory by every wave, the same rows went through
 // the L2 four times and that traffic, not the matrix pipe, set the pace.  u8 rows are dequantised on the way into
-// LDS ((code - zero-point) * scale, rounded to f16), rows beyond the context are written as zeros.  Query rows go
-// global -> registers per wave (each wave has its own), one stage ahead.  Within a stage lane (n, g) supplies channels 16 g .. 16 g + 15 of row n as the k-slices
-// of two matrix instructions (which channel sits in which k-slice is free as long as both operands agree).
+// LDS ((code - zero-point) * scale, rounded to f16), rows beyond the context are written as zeros.  Each wave's 32 query
+// rows take the same way into an LDS buffer of the wave's own, eight lanes to a row's 128 bytes (loaded straight
+// into operand layout -- sixteen rows per instruction, every lane in a cache line of its own -- the address unit set
+// the pace).  Within a stage lane (n, g) supplies channels 16 g .. 16 g + 15 of row n as the k-slices of two matrix
+// instructions (which channel sits in which k-slice is free as long as both operands agree).
 template <int D, int DT, int QDT, bool U8>
 __global__ __launch_bounds__(256, 2) void xatt_logits_kernel(XattArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");

@@ -8,23 +8,23 @@
 //   A  = mean over kv heads of S
 //   out[rb][c] = - sum over the 32 rows r of block rb of A[r][c]         [ev / 32, ev] values per sequence
 //
-// Four kernels.  The first three are O(ev * D) preparation, a wave per token row at a time:
+// Four kernels.  The first three are O(ev * D) preparation, sixteen lanes per token row:
 //   rkv_stats_colsum_kernel : per (head, token) the factor that normalises the row, and for u8 rows the zero-point
 //                       and the sum of the codes; the sum of the unit rows over chunks of 256 tokens (fixed order);
 //   rkv_total_kernel  : the chunks' sums added up in chunk order;
 //   rkv_mean_kernel   : row mean of S with its diagonal zeroed = (k^_r . sum_c k^_c - k^_r . k^_r) / ev, which
 //                       costs a dot product per row instead of a pass over the similarity matrix.
-// rkv_diversity_kernel is the O(ev^2 * D) part: a wave owns one 32-row block and 64 columns, loads the rows and
-// columns of one kv head straight into MFMA operands (lane (n, g): token 16 t + n, channels 32 s + 8 g .. + 7), forms
-// the 32 x 64 tile of raw dot products with v_mfma_f32_16x16x32_{f16,bf16}, scales / masks it in registers and
-// adds the rows up; heads accumulate in registers, so every output value is written once, by one lane, in a
-// fixed order (no atomics).
+// rkv_diversity_kernel is the O(ev^2 * D) part: a wave owns 32-row blocks and 64 columns, holds the columns of one kv
+// head as MFMA operands (lane (n, g): token 16 t + n, channels 32 s + 8 g .. + 7) and reads the rows, which its
+// workgroup shares, from LDS; it forms the 32 x 64 tiles of raw dot products with v_mfma_f32_16x16x32_{f16,bf16},
+// scales / masks them in registers and adds the rows up; heads accumulate in registers, so every output value is
+// written once, by one lane, in a fixed order (no atomics).
 // u8 caches: the codes are multiplied exactly as f16 subnormals (code * 2^-24, products summed in f32 without
 // rounding: at most 128 * 255^2 < 2^24), and scale / zero-point enter on the accumulator:
 //   k_r . k_c = sc_r sc_c (sum(c_r c_c) - zp_c sum(c_r) - zp_r sum(c_c) + D zp_r zp_c).
 //
 // Roofline: dense MFMA (2 * D flops per token pair and head); the operand rows come from L2 (every row is read
-// by ev / 64 waves as a row and ev / 128 or ev / 32 waves as a column).
+// by ev / 256 workgroups as a row and ev / 128 or ev / 32 waves as a column).
 #include "pa_device.h"
 
 namespace pa {
@@ -47,72 +47,100 @@ __device__ __forceinline__ f4 mma(const s8v& a, const s8v& b, const f4& c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
 }
 
-template <int D, int KVDT>
-__device__ __forceinline__ const uint8_t* token_row(const RkvDivArgs& a, const RkvDivSeq& q, int h, int j) {
-    constexpr int CROWB = KVDT == DT_U8 ? D + 8 : D * 2;
-    const int32_t phys = a.block_indices[q.table_off + q.first_block + (j >> 5)];
-    return a.key_cache + (((long)phys * a.Hkv + h) * 32 + (j & 31)) * CROWB;
+// Sum over the 16 lanes of a row (four cross-lane steps, the same order on every lane's side of each step).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+    v += dpp_f<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+    v += dpp_f<0x141>(v);  // row_half_mirror: the other quad of the eight
+    return v + dpp_f<0x140>(v);  // row_mirror: the other eight of the sixteen
 }
 
-// The lane's D / 64 channels of a row as floats (u8: dequantised), and for u8 the codes themselves.
+// The preparation kernels give a token row to 16 lanes, D / 16 consecutive channels each (8 or 16 bytes per lane at
+// D = 128), four rows per wave and load.  The lane's channels as floats (u8: dequantised), and for u8 the codes.
 template <int D, int KVDT>
-__device__ __forceinline__ void lane_channels(const uint8_t* row, int lane, float (&x)[D / 64], float (&code)[D / 64]) {
-    constexpr int EPL = D / 64;
+__device__ __forceinline__ void lane_channels(const uint8_t* row, int l16, float (&x)[D / 16], float (&code)[D / 16]) {
+    constexpr int E = D / 16;
     if (KVDT == DT_U8) {
         const float2 hd = *reinterpret_cast<const float2*>(row);
+        uint32_t w[E / 4];
+        if constexpr (E == 8) {
+            const u2v v = *reinterpret_cast<const u2v*>(row + 8 + 8 * l16);
+            w[0] = v[0];
+            w[1] = v[1];
+        } else {
+            w[0] = *reinterpret_cast<const uint32_t*>(row + 8 + 4 * l16);
+        }
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            code[e] = (float)row[8 + lane * EPL + e];
+        for (int e = 0; e < E; ++e) {
+            code[e] = (float)((w[e / 4] >> (8 * (e % 4))) & 0xffu);
             x[e] = (code[e] - hd.y) * hd.x;
         }
     } else {
-        const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
+        uint32_t w[E / 2];
+        if constexpr (E == 8) {
+            const u4v v = *reinterpret_cast<const u4v*>(row + 16 * l16);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
+            for (int i = 0; i < 4; ++i) w[i] = v[i];
+        } else {
+            const u2v v = *reinterpret_cast<const u2v*>(row + 8 * l16);
+            w[0] = v[0];
+            w[1] = v[1];
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
             code[e] = 0.0f;
-            x[e] = KVDT == DT_F16 ? half_bits_to_float(r16[lane * EPL + e]) : bf16_bits_to_float(r16[lane * EPL + e]);
+            x[e] = load16<KVDT>((uint16_t)(w[e / 2] >> (16 * (e % 2))));
         }
     }
 }
 
-// One pass over the area's rows, a workgroup per (sequence, head, chunk of 256 tokens), a wave per token at a time:
+// One pass over the area's rows, a workgroup per (sequence, head, chunk of 256 tokens):
 //   stats[h][token] = { factor that turns the raw dot product of two rows into their cosine (1 / |k|, times the
 //                       row's scale for u8), zero-point, sum of codes, k^ . k^ }
-//   colsum[seq][h][chunk][d] = sum of k^[d] over the chunk's tokens: wave w adds tokens w, w + 4, ... in order, the
-//                       four waves' sums are added in wave order.
+//   colsum[seq][h][chunk][d] = sum of k^[d] over the chunk's tokens: each of the workgroup's sixteen 16-lane groups
+//                       adds tokens group, group + 16, ... in order, the groups' sums are added in group order.
 template <int D, int KVDT>
 __global__ __launch_bounds__(256) void rkv_stats_colsum_kernel(RkvDivArgs a) {
-    constexpr int EPL = D / 64;
-    __shared__ float red[4][D];
+    constexpr int E = D / 16;
+    __shared__ float red[16][D];
     const RkvDivSeq q = a.seqs[blockIdx.z];
     const int h = blockIdx.y;
     const int base = blockIdx.x * CHUNK;
     if (base >= q.ev) return;
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    float acc[EPL];
+    const int l16 = threadIdx.x & 15, grp = threadIdx.x >> 4;
+    float acc[E];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
-#pragma unroll 8
-    for (int i = 0; i < CHUNK / 4; ++i) {
-        const int j = base + w + 4 * i;
+    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    constexpr int CROWB = KVDT == DT_U8 ? D + 8 : D * 2;
+    const int32_t* table = a.block_indices + q.table_off + q.first_block;
+    const int last_blk = q.ev / 32 - 1;
+#pragma unroll 4
+    for (int i = 0; i < CHUNK / 16; ++i) {
+        const int j = base + grp + 16 * i;
         const bool live = j < q.ev;
-        // rows beyond the area repeat its last one: the loads are unconditional, so that an unrolled round's loads
-        // are in flight together; such rows add zeros and write nothing
-        const uint8_t* row = token_row<D, KVDT>(a, q, h, min(j, q.ev - 1));
-        float x[EPL], code[EPL];
-        lane_channels<D, KVDT>(row, lane, x, code);
+        // rows beyond the area repeat a row of its last block: the loads are unconditional, so that an unrolled round's
+        // loads are in flight together; such rows add zeros and write nothing.  (The block is the same for the whole
+        // workgroup: base is a multiple of 32 and grp below 16, so its id is read once, by the scalar unit.)
+        const int32_t phys = table[min(base / 32 + (i >> 1), last_blk)];
+        const uint8_t* row = a.key_cache + (((long)phys * a.Hkv + h) * 32 + (grp + 16 * (i & 1))) * CROWB;
+        float x[E], code[E];
+        lane_channels<D, KVDT>(row, l16, x, code);
         float sq = 0.0f, cs = 0.0f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
+        for (int e = 0; e < E; ++e) {
             sq = fmaf(x[e], x[e], sq);
             cs += code[e];
         }
-        sq = wave_sum(sq);
-        cs = wave_sum(cs);  // integers below 2^24: exact in any order
+        sq = row16_sum(sq);
+        cs = row16_sum(cs);  // integers below 2^24: exact in any order
         const float inv = 1.0f / sqrtf(sq + NORM_EPS);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] += live ? x[e] * inv : 0.0f;
-        if (lane == 0 && live) {
+        for (int e = 0; e < E; ++e) acc[e] += live ? x[e] * inv : 0.0f;
+        if (l16 == 0 && live) {
             float sc = 1.0f, zp = 0.0f;
             if (KVDT == DT_U8) {
                 const float2 hd = *reinterpret_cast<const float2*>(row);
@@ -123,10 +151,12 @@ __global__ __launch_bounds__(256) void rkv_stats_colsum_kernel(RkvDivArgs a) {
         }
     }
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) red[w][lane * EPL + e] = acc[e];
+    for (int e = 0; e < E; ++e) red[grp][l16 * E + e] = acc[e];
     __syncthreads();
     if (threadIdx.x < D) {
-        const float s = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+        float s = red[0][threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < 16; ++k) s += red[k][threadIdx.x];
         a.colsum[(((long)blockIdx.z * a.Hkv + h) * (a.chunks_max + 1) + 1 + blockIdx.x) * D + threadIdx.x] = s;
     }
 }
@@ -144,77 +174,101 @@ __global__ __launch_bounds__(D) void rkv_total_kernel(RkvDivArgs a) {
 }
 
 // mean[h][token] = (k^_r . sum over the area's tokens of k^ - k^_r . k^_r) / ev, divided by the row's factor; a
-// wave takes eight tokens, whose loads go out together.
+// workgroup takes 128 tokens, each 16-lane group eight of them, whose loads go out together.
 template <int D, int KVDT>
 __global__ __launch_bounds__(256) void rkv_mean_kernel(RkvDivArgs a) {
-    constexpr int EPL = D / 64;
-    constexpr int TPW = 8;
+    constexpr int E = D / 16;
+    constexpr int TPG = 8;
     const RkvDivSeq q = a.seqs[blockIdx.z];
     const int h = blockIdx.y;
-    const int j0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * TPW;
-    if (j0 >= q.ev) return;
-    const int lane = threadIdx.x & 63;
+    const int l16 = threadIdx.x & 15, grp = threadIdx.x >> 4;
+    const int j0 = blockIdx.x * (16 * TPG) + grp;   // tokens j0, j0 + 16, ..
+    if (blockIdx.x * (16 * TPG) >= q.ev) return;
     const float* tot = a.colsum + ((long)blockIdx.z * a.Hkv + h) * (a.chunks_max + 1) * D;
-    float s[EPL];
+    float s[E];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) s[e] = tot[lane * EPL + e];
-    float dot[TPW], self[TPW], fac[TPW];
+    for (int e = 0; e < E; ++e) s[e] = tot[l16 * E + e];
+    constexpr int CROWB = KVDT == DT_U8 ? D + 8 : D * 2;
+    const int32_t* table = a.block_indices + q.table_off + q.first_block;
+    const int last_blk = q.ev / 32 - 1;
+    float dot[TPG], self[TPG], fac[TPG];
 #pragma unroll
-    for (int t = 0; t < TPW; ++t) {
-        const int j = min(j0 + t, q.ev - 1);
+    for (int t = 0; t < TPG; ++t) {
+        // (tokens beyond the area: a row of its last block, nothing is written for them; the block is the same for the
+        // whole workgroup, so its id is read by the scalar unit)
+        const int blk = min(blockIdx.x * (TPG / 2) + (t >> 1), last_blk);
+        const int j = blk * 32 + grp + 16 * (t & 1);
         const float4 st = a.stats[(long)h * a.total_tok + q.tok_off + j];
-        const uint8_t* row = token_row<D, KVDT>(a, q, h, j);
-        float x[EPL], code[EPL];
-        lane_channels<D, KVDT>(row, lane, x, code);
+        const uint8_t* row = a.key_cache + (((long)table[blk] * a.Hkv + h) * 32 + (grp + 16 * (t & 1))) * CROWB;
+        float x[E], code[E];
+        lane_channels<D, KVDT>(row, l16, x, code);
         float d = 0.0f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) d = fmaf(KVDT == DT_U8 ? (code[e] - st.y) * st.x : x[e] * st.x, s[e], d);
+        for (int e = 0; e < E; ++e) d = fmaf(KVDT == DT_U8 ? (code[e] - st.y) * st.x : x[e] * st.x, s[e], d);
         dot[t] = d;
         self[t] = st.w;
         fac[t] = st.x;
     }
 #pragma unroll
-    for (int t = 0; t < TPW; ++t) dot[t] = wave_sum(dot[t]);
-    if (lane == 0) {
+    for (int t = 0; t < TPG; ++t) dot[t] = row16_sum(dot[t]);
+    if (l16 == 0) {
 #pragma unroll
-        for (int t = 0; t < TPW; ++t)
-            if (j0 + t < q.ev)  // stored over the row's factor: what the raw product times the column's factor is held against
-                a.mean[(long)h * a.total_tok + q.tok_off + j0 + t] = (dot[t] - self[t]) / (float)q.ev / fac[t];
+        for (int t = 0; t < TPG; ++t)
+            if (j0 + 16 * t < q.ev)  // stored over the row's factor: what the raw product times the column's factor is held against
+                a.mean[(long)h * a.total_tok + q.tok_off + j0 + 16 * t] = (dot[t] - self[t]) / (float)q.ev / fac[t];
     }
 }
 
-// DT: MFMA operand type (f16 for f16 and u8 caches, bf16 for bf16 caches).  RB: 32-row blocks per wave -- the
-// wave's 64 columns stay in registers while it walks RB row blocks, so a large area reads each operand row from L2
-// fewer times; small areas use RB = 1 to have enough waves.
+// DT: MFMA operand type (f16 for f16 and u8 caches, bf16 for bf16 caches).  RB: 32-row blocks per workgroup.
+// A workgroup owns RB row blocks and 256 columns, 64 to a wave.  Per kv head the rows of its RB blocks and their
+// per-row terms go global -> registers -> LDS once (coalesced: a row block of one head is contiguous in the cache) and
+// serve all four waves; the wave's 64 columns stay in registers for the head.  (With every wave loading rows and
+// per-row terms straight into operand layout, 9 KB per 16 matrix instructions came back through the vector memory
+// path, which then set the pace: 15 % of the matrix peak.)  The next head's rows are asked for before the current
+// head's arithmetic and written to LDS behind it.
+// LDS rows hold operands: 2 D bytes (u8 codes widened to 16 bits on the way in, once per workgroup instead of once
+// per wave and use) + 16 bytes of padding (the 16-byte operand reads of sixteen rows touch every bank).
+template <int D, bool U8, int RB>
+struct RkvTile {
+    static constexpr int CROWB = U8 ? D + 8 : D * 2;
+    static constexpr int ROWS = RB * 32;
+    static constexpr int LROW = D * 2 + 16;
+    static constexpr int BLKB = 32 * LROW;                 // LDS bytes of one row block
+    static constexpr int PIECES = 32 * D / 8;              // pieces (eight channels: 8 bytes of codes, or 16 bytes) of a (block, head)
+    static constexpr int PPT = (PIECES + 255) / 256;       // pieces per thread and row block
+    static constexpr int OPB = RB * BLKB;
+    static constexpr int LDSB = OPB + ROWS * 16;           // operands | per-row terms {factor, zero-point, code sum, threshold}
+};
+
 template <int D, int DT, bool U8, int RB>
 __global__ __launch_bounds__(256) void rkv_diversity_kernel(RkvDivArgs a) {
+    using T = RkvTile<D, U8, RB>;
     constexpr int KS = D / 32;
+    constexpr int CROWB = T::CROWB;
     constexpr float CODE_UNIT2 = 281474976710656.0f;  // 2^48: both operands are code * 2^-24
+    __shared__ __align__(16) uint8_t lds[T::LDSB];
     const RkvDivSeq q = a.seqs[blockIdx.z];
     const int rb0 = blockIdx.y * RB;
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    if (rb0 * 32 >= q.ev || blockIdx.x * 256 >= q.ev) return;  // (the whole workgroup)
     const int col0 = (blockIdx.x * 4 + wv) * 64;
-    if (rb0 * 32 >= q.ev || col0 >= q.ev) return;
+    const bool wave_live = col0 < q.ev;  // a wave beyond the area still moves rows and meets the barriers
     const int n = lane & 15, g = lane >> 4;
     const int last_rb = q.ev / 32 - 1;
 
-    // physical blocks of the wave's column tokens and row tokens, looked up once for all heads
-    constexpr int CROWB = U8 ? D + 8 : D * 2;
+    // physical blocks of the wave's column tokens and of the workgroup's row blocks, looked up once for all heads
     const int32_t* table = a.block_indices + q.table_off + q.first_block;
-    long col_off[4], row_off[RB][2];
+    long col_off[4], blk_off[RB];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const int j = min(col0 + 16 * c + n, q.ev - 1);  // columns beyond the area repeat its last token
         col_off[c] = ((long)table[j >> 5] * a.Hkv * 32 + (j & 31)) * CROWB;
     }
 #pragma unroll
-    for (int k = 0; k < RB; ++k) {
-        const int rb = min(rb0 + k, last_rb);  // row blocks beyond the area repeat its last one
-        const long blk = (long)table[rb] * a.Hkv * 32;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) row_off[k][t] = (blk + 16 * t + n) * CROWB;
-    }
-    auto operand = [&](int h, long off, s8v (&reg)[KS]) {
+    for (int k = 0; k < RB; ++k)  // row blocks beyond the area repeat its last one; their sums are never written
+        blk_off[k] = (long)table[min(rb0 + k, last_rb)] * a.Hkv * 32 * CROWB;
+
+    auto col_operand = [&](int h, long off, s8v (&reg)[KS]) __attribute__((always_inline)) {
         const uint8_t* row = a.key_cache + off + (long)h * 32 * CROWB;
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -229,6 +283,50 @@ __global__ __launch_bounds__(256) void rkv_diversity_kernel(RkvDivArgs a) {
             reg[s] = __builtin_bit_cast(s8v, v);
         }
     };
+    // a head's rows and per-row terms on their way to LDS: thread tid moves pieces tid, tid + 256, .. of every row
+    // block and the terms of row tid
+    constexpr int PPR = D / 8;  // pieces per row
+    struct Staged {
+        u4v piece[RB][T::PPT];  // (u8: the first two words)
+        float4 terms;
+    };
+    auto fetch = [&](Staged& sg, int h) __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            const uint8_t* src = a.key_cache + blk_off[k] + (long)h * 32 * CROWB;
+#pragma unroll
+            for (int i = 0; i < T::PPT; ++i) {
+                const int p = min(tid + 256 * i, T::PIECES - 1);
+                if (U8) {
+                    const u2v cd = *reinterpret_cast<const u2v*>(src + (p / PPR) * CROWB + 8 + 8 * (p % PPR));
+                    sg.piece[k][i] = u4v{cd[0], cd[1], 0u, 0u};
+                } else {
+                    sg.piece[k][i] = *reinterpret_cast<const u4v*>(src + 16 * p);
+                }
+            }
+        }
+        if (tid < T::ROWS) {
+            const long r = (long)h * a.total_tok + q.tok_off + min(rb0 + (tid >> 5), last_rb) * 32 + (tid & 31);
+            const float4 st = a.stats[r];
+            sg.terms = make_float4(st.x, st.y, st.z * (1.0f / CODE_UNIT2), a.mean[r]);
+        }
+    };
+    auto put = [&](const Staged& sg) __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < RB; ++k)
+#pragma unroll
+            for (int i = 0; i < T::PPT; ++i) {
+                const int p = tid + 256 * i;
+                if (p < T::PIECES) {
+                    u4v v = sg.piece[k][i];
+                    if (U8)  // code bytes to 16-bit words: code * 2^-24 as f16
+                        v = u4v{__builtin_amdgcn_perm(0u, v[0], 0x0c010c00u), __builtin_amdgcn_perm(0u, v[0], 0x0c030c02u),
+                                __builtin_amdgcn_perm(0u, v[1], 0x0c010c00u), __builtin_amdgcn_perm(0u, v[1], 0x0c030c02u)};
+                    *reinterpret_cast<u4v*>(lds + k * T::BLKB + (p / PPR) * T::LROW + 16 * (p % PPR)) = v;
+                }
+            }
+        if (tid < T::ROWS) *reinterpret_cast<float4*>(lds + T::OPB + 16 * tid) = sg.terms;
+    };
 
     // Per element the vector unit does little: with raw = the accumulator, a_r / a_c the rows' factors and m_r the
     // row mean,
@@ -241,12 +339,17 @@ __global__ __launch_bounds__(256) void rkv_diversity_kernel(RkvDivArgs a) {
     for (int k = 0; k < RB; ++k)
 #pragma unroll
         for (int c = 0; c < 4; ++c) colacc[k][c] = 0.0f;
+    Staged sg;
+    fetch(sg, 0);
+    put(sg);
+    __syncthreads();
     for (int h = 0; h < a.Hkv; ++h) {
         const long sbase = (long)h * a.total_tok + q.tok_off;
+        if (h + 1 < a.Hkv) fetch(sg, h + 1);
         s8v breg[4][KS];
         // (no branch around the loads of columns beyond the area; they are never written)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) operand(h, col_off[c], breg[c]);
+        for (int c = 0; c < 4; ++c) col_operand(h, col_off[c], breg[c]);
         float c_fac[4], c_zp[4], c_w[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -255,42 +358,49 @@ __global__ __launch_bounds__(256) void rkv_diversity_kernel(RkvDivArgs a) {
             c_zp[c] = st.y;
             c_w[c] = (st.z - (float)D * st.y) * (1.0f / CODE_UNIT2);
         }
+        if (wave_live) {
 #pragma unroll
-        for (int k = 0; k < RB; ++k) {
-            const int rb = min(rb0 + k, last_rb);  // the sums of repeated blocks are never written
-            s8v areg[2][KS];
+            for (int k = 0; k < RB; ++k) {
+                const int rb = min(rb0 + k, last_rb);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) operand(h, row_off[k][t], areg[t]);
+                for (int t = 0; t < 2; ++t) {
+                    s8v areg[KS];
+                    const uint8_t* row = lds + k * T::BLKB + (16 * t + n) * T::LROW;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                float r_fac[4], r_thr[4], r_zp[4], r_cs[4];
+                    for (int s = 0; s < KS; ++s)
+                        areg[s] = __builtin_bit_cast(s8v, *reinterpret_cast<const u4v*>(row + (32 * s + 8 * g) * 2));
+                    float4 rt[4];  // {factor, zero-point, code sum, threshold} of rows 16 t + 4 g + i
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int r = rb * 32 + 16 * t + 4 * g + i;
-                    const float4 st = a.stats[sbase + r];
-                    r_fac[i] = st.x;
-                    r_thr[i] = a.mean[sbase + r];
-                    r_zp[i] = st.y;
-                    r_cs[i] = st.z * (1.0f / CODE_UNIT2);
-                }
+                    for (int i = 0; i < 4; ++i)
+                        rt[i] = *reinterpret_cast<const float4*>(lds + T::OPB + 16 * (32 * k + 16 * t + 4 * g + i));
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    f4 acc = f4{0.0f, 0.0f, 0.0f, 0.0f};
+                    for (int c = 0; c < 4; ++c) {
+                        f4 acc = f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                    for (int s = 0; s < KS; ++s) acc = mma<DT>(areg[t][s], breg[c][s], acc);
-                    const bool diag_tile = rb * 32 + 16 * t == col0 + 16 * c;
+                        for (int s = 0; s < KS; ++s) acc = mma<DT>(areg[s], breg[c][s], acc);
+                        float v[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        float raw = acc[i];
-                        if (U8) raw = fmaf(-r_zp[i], c_w[c], fmaf(-c_zp[c], r_cs[i], raw));
-                        float v = raw * c_fac[c];
-                        if (diag_tile && 4 * g + i == n) v = 0.0f;
-                        colacc[k][c] = fmaf(v < r_thr[i] ? 0.0f : v, r_fac[i], colacc[k][c]);
+                        for (int i = 0; i < 4; ++i) {
+                            float raw = acc[i];
+                            if (U8) raw = fmaf(-rt[i].y, c_w[c], fmaf(-c_zp[c], rt[i].z, raw));
+                            v[i] = raw * c_fac[c];
+                        }
+                        if (rb * 32 + 16 * t == col0 + 16 * c) {  // (uniform) the tile that holds the diagonal
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                if (4 * g + i == n) v[i] = 0.0f;
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) colacc[k][c] = fmaf(v[i] < rt[i].w ? 0.0f : v[i], rt[i].x, colacc[k][c]);
                     }
                 }
             }
         }
+        __syncthreads();  // every wave is done with this head's rows
+        if (h + 1 < a.Hkv) put(sg);
+        __syncthreads();
     }
+    if (!wave_live) return;
     const float inv_h = 1.0f / (float)a.Hkv;
 #pragma unroll
     for (int k = 0; k < RB; ++k) {
@@ -314,7 +424,7 @@ hipError_t launch_typed(hipStream_t s, const RkvDivArgs& a, int nseq, int ev_max
     hipLaunchKernelGGL((rkv_stats_colsum_kernel<D, KVDT>), dim3((unsigned)chunks, (unsigned)a.Hkv, (unsigned)nseq), block, 0,
                        s, a);
     hipLaunchKernelGGL((rkv_total_kernel<D>), dim3((unsigned)a.Hkv, (unsigned)nseq), dim3(D), 0, s, a);
-    hipLaunchKernelGGL((rkv_mean_kernel<D, KVDT>), dim3((unsigned)ceil_div(ev_max, 32), (unsigned)a.Hkv, (unsigned)nseq),
+    hipLaunchKernelGGL((rkv_mean_kernel<D, KVDT>), dim3((unsigned)ceil_div(ev_max, 128), (unsigned)a.Hkv, (unsigned)nseq),
                        block, 0, s, a);
     // four row blocks per wave once that still leaves a few thousand waves
     const long waves4 = (long)nseq * ceil_div(ev_max, 128) * ceil_div(ev_max, 64);

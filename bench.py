@@ -61,6 +61,9 @@ def parse():
     ap.add_argument("--xattention", type=float, default=0.0, metavar="THRESHOLD",
                     help="adds a leg: block-sparse prefill with this threshold against dense prefill (4 x 512-token "
                          "chunks, Qwen2.5-7B shape, bf16 cache)")
+    ap.add_argument("--rotate", action="store_true",
+                    help="adds a leg: cache rotation (the re-rotation of K rows behind evicted blocks) over every "
+                         "block of the workload's sequences, one layer")
     ap.add_argument("--kv-cache-leg", action="store_true",
                     help="adds a leg: copy-on-write of 256 blocks x 32 layers and growth of the cache tensors")
     ap.add_argument("--pool-factor", type=float, default=2.0,
@@ -278,6 +281,35 @@ def diversity_leg(torch, op, spec, kc, dev, ev, reps=20):
             "note": "2 * D flops per (token pair, kv head); wall time of the whole call (four kernels, one upload)"}
 
 
+def rotation_leg(torch, pkg, op, spec, kc, dev, reps=10):
+    """Cache rotation of every block of the workload's sequences (one layer, one delta per block): wall time of
+    the whole call (argument checks, one upload of the block list and deltas, two stream waits, one kernel),
+    events on the launch stream.  Rotates a copy of the K cache, in place."""
+    Hkv, D, bs = spec["Hkv"], spec["D"], spec["bs"]
+    blocks = np.ascontiguousarray(spec["block_indices"], np.int32)
+    rng = np.random.default_rng(77)
+    max_blocks = 512
+    deltas = rng.integers(1, max_blocks, size=(len(blocks), 1)).astype(np.int32)
+    op.set_rotation_trig_lut(pkg.rotation_trig_lut(bs, max_blocks, D))
+    work = kc.clone()
+    for _ in range(2):
+        op.rotate_cache(work, blocks, deltas)
+    torch.cuda.synchronize(dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        op.rotate_cache(work, blocks, deltas)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    ms = e0.elapsed_time(e1) / reps
+    row = D + 8 if spec["kv_dtype"] == "u8" else 2 * D
+    nbytes = 2.0 * len(blocks) * Hkv * bs * row
+    return {"blocks": int(len(blocks)), "ms_per_call": round(ms, 4), "bytes": nbytes,
+            "roofline": {"bound": "hbm", "kernel": "pa_rotate_rows_kernel", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+            "note": "every K row read and written once; wall time of the whole call"}
+
+
 def xattention_leg(torch, pkg, dev, threshold, kv_dtype="bf16", reps=20):
     """Block-sparse prefill (XAttention, block 64, stride 8) against dense prefill on the prefill part of the mixed
     workload: four 512-token chunks at past 0 / 2048 / 4096 / 8192, Qwen2.5-7B shape, bf16 cache (u8 with --kv-dtype u8).  Plain N(0,1) data
@@ -487,6 +519,8 @@ def main():
         res["xattention"] = xattention_leg(torch, pkg, dev, args.xattention, "u8" if args.kv_dtype == "u8" else "bf16")
     if args.diversity > 0:
         res["adaptive_rkv_diversity"] = diversity_leg(torch, op, spec, kc, dev, args.diversity)
+    if args.rotate:
+        res["cache_rotation"] = rotation_leg(torch, pkg, op, spec, kc, dev)
     if args.kv_cache_leg:
         res["kv_cache"] = kv_cache_leg(torch, pkg, dev)
     if args.config == 4:

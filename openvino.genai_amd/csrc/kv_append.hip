@@ -17,23 +17,6 @@ namespace {
 // takes four consecutive tokens of one kv head, so that what it writes is one run of cache bytes wherever the
 // tokens share a block.  Minimum and maximum of a row are reduced over its 16 lanes with four
 // cross-lane (DPP) steps; the arithmetic per element is that of quantize_row_u8, so the bytes are the same.
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float row16_min(float v) {
-    v = fminf(v, dpp_f<0xB1>(v));   // quad_perm [1, 0, 3, 2]
-    v = fminf(v, dpp_f<0x4E>(v));   // quad_perm [2, 3, 0, 1]
-    v = fminf(v, dpp_f<0x141>(v));  // row_half_mirror: the other quad of the eight
-    return fminf(v, dpp_f<0x140>(v));  // row_mirror: the other eight of the sixteen
-}
-__device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, dpp_f<0xB1>(v));
-    v = fmaxf(v, dpp_f<0x4E>(v));
-    v = fmaxf(v, dpp_f<0x141>(v));
-    return fmaxf(v, dpp_f<0x140>(v));
-}
-
 template <int QDT, int KVDT, int E>
 __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ key,
                                                         const uint16_t* __restrict__ value,

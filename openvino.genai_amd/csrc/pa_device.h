@@ -55,6 +55,42 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
+// ---- reductions over the 16 lanes of a row (a row of a DPP row: lanes 16 k .. 16 k + 15) ----------------------
+// Four cross-lane steps each; every lane ends up with the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_min(float v) {
+    v = fminf(v, dpp_f<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+    v = fminf(v, dpp_f<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+    v = fminf(v, dpp_f<0x141>(v));  // row_half_mirror: the other quad of the eight
+    return fminf(v, dpp_f<0x140>(v));  // row_mirror: the other eight of the sixteen
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    v = fmaxf(v, dpp_f<0x141>(v));
+    return fmaxf(v, dpp_f<0x140>(v));
+}
+// ... and over the 8 lanes of a half row
+__device__ __forceinline__ float row8_min(float v) {
+    v = fminf(v, dpp_f<0xB1>(v));
+    v = fminf(v, dpp_f<0x4E>(v));
+    return fminf(v, dpp_f<0x141>(v));
+}
+__device__ __forceinline__ float row8_max(float v) {
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    return fmaxf(v, dpp_f<0x141>(v));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    return v + dpp_f<0x140>(v);
+}
+
 // ---- one K or V row into a u8 cache row ---------------------------------------------------------
 // A 64-lane wave quantises one row of D = 64 * EPL elements: `f32 scale | f32 zero-point | D codes` with
 //   scale = (max - min) / 255  (a zero range takes 1e-4),  zp = -min / scale,

@@ -47,18 +47,6 @@ __device__ __forceinline__ f4 mma(const s8v& a, const s8v& b, const f4& c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
 }
 
-// Sum over the 16 lanes of a row (four cross-lane steps, the same order on every lane's side of each step).
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float row16_sum(float v) {
-    v += dpp_f<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-    v += dpp_f<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-    v += dpp_f<0x141>(v);  // row_half_mirror: the other quad of the eight
-    return v + dpp_f<0x140>(v);  // row_mirror: the other eight of the sixteen
-}
-
 // The preparation kernels give a token row to 16 lanes, D / 16 consecutive channels each (8 or 16 bytes per lane at
 // D = 128), four rows per wave and load.  The lane's channels as floats (u8: dequantised), and for u8 the codes.
 template <int D, int KVDT>

@@ -54,6 +54,28 @@ def test_rotate_cache_bit_exact(pkg, dev, kd, D, per_token):
     assert np.array_equal(kc.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("kd,D", [("u8", 128), ("bf16", 128), ("f16", 64), ("u8", 64)])
+def test_rotate_cache_row_count_not_a_multiple_of_a_workgroup(pkg, dev, kd, D):
+    """16-token blocks, one kv head, three blocks: 48 rows, so the kernel's last workgroup is half empty."""
+    import torch
+    print(f"case rotate ragged {kd} D={D}", flush=True)
+    rng = np.random.default_rng(22)
+    nb, Hkv, bs = 9, 1, 16
+    cache = _random_cache(rng, nb, Hkv, bs, D, kd)
+    lut = pkg.rotation_trig_lut(bs, 32, D, 10000.0)
+    blocks = np.array([7, 0, 4], np.int32)
+    deltas = rng.integers(1, 32, size=(3, bs)).astype(np.int32)
+    ref = cache.copy()
+    O.rotate_cache(ref, H.DT[kd], blocks, deltas, lut)
+    qd = "f16" if kd == "u8" else kd
+    op = pkg.PagedAttention(4, Hkv, D, bs, qd, kd, device=0, stream=torch.cuda.current_stream(dev))
+    op.set_rotation_trig_lut(lut)
+    kc = torch.from_numpy(cache).to(dev)
+    op.rotate_cache(kc, blocks, deltas)
+    op.synchronize()
+    assert np.array_equal(kc.cpu().numpy(), ref)
+
+
 def test_rotate_cache_rejects_bad_arguments(pkg, dev):
     import torch
     op = pkg.PagedAttention(8, 2, 128, 32, "f16", "u8", device=0, stream=torch.cuda.current_stream(dev))

@@ -62,6 +62,18 @@ def test_diversity_matches_checker(pkg, kv, q, D):
     assert max(np.abs(r).max() for _, r in res) > 1.0
 
 
+@pytest.mark.parametrize("kv,q,D", [("u8", "f16", 128), ("bf16", "bf16", 64), ("f16", "f16", 128)])
+def test_diversity_of_long_areas(pkg, kv, q, D):
+    """Areas long enough for the launch that gives a workgroup four row blocks (the one the benchmark measures): a
+    whole number of 128-row groups, an area whose last group holds one block and whose last 256 columns hold 32, and
+    a short one beside them."""
+    print(f"case diversity long {kv} D={D}", flush=True)
+    lens = [4200, 2200, 500, 130]
+    ev = [4096, 2080, 0, 96]
+    got, res = _run(pkg, kv, q, 4, 2, D, lens, 32, ev, seed=31 + D)
+    assert len(res) == 3
+
+
 @pytest.mark.parametrize("Hkv", [1, 4, 8])
 def test_diversity_over_kv_head_counts(pkg, Hkv):
     _run(pkg, "u8", "f16", 8, Hkv, 128, [600, 300], 32, [512, 256], seed=Hkv)

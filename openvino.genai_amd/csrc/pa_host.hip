@@ -383,7 +383,7 @@ void plan_items(pa_ctx* ctx) {
     // 16-bit caches: every dense item goes to the narrow kernel variant (128 query rows per workgroup, four waves per
     // SIMD), which outruns the wide one there; u8 caches need the wide variant's registers
     const bool narrow_all = ctx->cfg.kv_cache_dtype != PA_U8;
-    const int32_t QT = std::max(1, (narrow_all ? 128 : 256) / G), QTX = std::max(1, 128 / G), sw = ctx->sliding_window;
+    const int32_t QT = std::max(1, 128 / G), QTX = std::max(1, 128 / G), sw = ctx->sliding_window;
     struct Tile { int32_t b, q0, nq, lo, hi, kind; };  // kind 0: more than 16 rows, 1: the rest, 2: single-token sequences, 3: block-sparse
     std::vector<int32_t> single_idx(B, -1);
     int32_t n_single_seqs = 0;

@@ -171,14 +171,16 @@ __device__ __forceinline__ void wait_vmem() {
 // that belongs at its LDS position.  With no
 // staging registers the kernel fits three waves per SIMD at two 16-row groups per wave: half the LDS operand traffic
 // per matrix instruction of the one-group variant.
-template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT, bool DMA>
-__global__ __launch_bounds__(DMA ? 256 : 512, DMA ? 2 : (PIPE || U8) ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
+template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT, bool DMA, bool HALF = false>
+__global__ __launch_bounds__((DMA || HALF) ? 256 : 512, (DMA || HALF) ? 2 : (PIPE || U8) ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
 void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     static_assert(!XATT || !PIPE, "the block-sparse variant works a block through in one go");
     static_assert(U8 || DT == QDT, "16-bit caches are used in the query's type");
     static_assert(!DMA || (!U8 && !PIPE && !XATT && D == 128), "the straight-to-LDS variant: dense items, 16-bit caches, head size 128");
-    constexpr int NT = DMA ? 256 : 512;
+    constexpr int NT = (DMA || HALF) ? 256 : 512;
+    constexpr int NCH = TOK * (D * 2 / 16);  // 16-byte chunks (eight codes of a u8 row) per block and tensor: 512 (D = 128) or 256 (D = 64)
+    constexpr int UPT = HALF ? NCH / NT : 1;  // load units (a chunk, or eight codes and a row header) per thread and tensor
     constexpr int ROWB = D * 2;            // bytes of a row as staged in LDS
     constexpr int CROWB = U8 ? D + 8 : D * 2;  // bytes of a row in the cache
     constexpr int LROWK = DMA ? ROWB : ROWB + 16;  // LDS row strides chosen so that the operand reads are bank-conflict free:
@@ -188,8 +190,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
     constexpr int KS = D / 32;
     constexpr int RT = D / 16;
     constexpr int CPR = ROWB / 16;         // 16-byte chunks per row
-    constexpr int NCH = TOK * CPR;         // chunks per block and tensor: 512 (D = 128) or 256 (D = 64)
-    static_assert(DMA || NCH <= NT, "one chunk per thread");
+    static_assert(DMA || NCH <= NT * UPT, "one chunk per load unit");
     constexpr int HDRB = U8 ? 4 * TOK * 4 : 0;  // per buffer: sc_k | zp_k * sc_k | sc_v | zp_v, one f32 per token each
     constexpr float CODE_UNIT = 16777216.0f;    // a code byte read as f16 is code * 2^-24
     // The loop works on three blocks at once (see the pipeline below): K of block t+1, V of block t-1 and the
@@ -319,11 +320,16 @@ void pa_prefill16_kernel(PrefillArgs a) {
     // three blocks in flight in registers.  16-bit cache: thread = one 16-byte chunk of K and of V per block.
     // u8 cache: thread = (row, group of 8 codes) plus the row's header; it writes the 8 codes as 16-bit words (16
     // bytes) -- same LDS address either way.  Threads beyond the chunk count repeat the loads of the first ones.
-    KvRegs<U8> set[3];
+    KvRegs<U8> set[HALF ? 2 : 3][UPT];
     const bool loader = tid < NCH;
     const int ltid = tid % NCH;
     const int lds_k = (ltid / CPR) * LROWK + (ltid % CPR) * 16;
     const int lds_v = OFF_V + (ltid / CPR) * LROWV + (ltid % CPR) * 16;
+    // (a thread's second load unit, where it has one: the chunk NT further on, i.e. the same piece of the row 16 below)
+    auto unit_loads = [&](int uu) __attribute__((always_inline)) { return uu == 0 ? loader : tid + NT * uu < NCH; };
+    auto unit_id = [&](int uu) __attribute__((always_inline)) { return uu == 0 ? ltid : (tid + NT * uu) % NCH; };
+    auto unit_lds_k = [&](int uu) __attribute__((always_inline)) { return uu == 0 ? lds_k : (unit_id(uu) / CPR) * LROWK + (unit_id(uu) % CPR) * 16; };
+    auto unit_lds_v = [&](int uu) __attribute__((always_inline)) { return uu == 0 ? lds_v : OFF_V + (unit_id(uu) / CPR) * LROWV + (unit_id(uu) % CPR) * 16; };
     const int kv_len = past + st.subsequence_begins[b + 1] - t0;
     // The kernel's tiles are 32 tokens: one 32-token cache block, or two 16-token blocks, in which case each row is
     // fetched from the block it lies in (a last tile of one block repeats it; those rows lie beyond kv_len).
@@ -338,24 +344,33 @@ void pa_prefill16_kernel(PrefillArgs a) {
         const long hi = ((long)table[min(2 * tile + 1, last_block16)] * Hkv + hkv) * (16 * CROWB) - 16 * CROWB;
         return upper ? hi : lo;
     };
-    auto fetch = [&](KvRegs<U8>& r, int j) __attribute__((always_inline)) {
-        const long blk = tile_base(tile_at(j), ltid / CPR >= 16);
-        if constexpr (U8) {
-            const long row = blk + (long)(ltid / CPR) * CROWB;
-            kv_issue(r, a.key_cache + row, a.value_cache + row, 8 + (ltid % CPR) * 8);
-        } else {
-            kv_issue(r, a.key_cache + blk + (long)ltid * 16, a.value_cache + blk + (long)ltid * 16);
+    auto fetch = [&](KvRegs<U8> (&rs)[UPT], int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int uu = 0; uu < UPT; ++uu) {
+            KvRegs<U8>& r = rs[uu];
+            const int lt = unit_id(uu);
+            const long blk = tile_base(tile_at(j), lt / CPR >= 16);
+            if constexpr (U8) {
+                const long row = blk + (long)(lt / CPR) * CROWB;
+                kv_issue(r, a.key_cache + row, a.value_cache + row, 8 + (lt % CPR) * 8);
+            } else {
+                kv_issue(r, a.key_cache + blk + (long)lt * 16, a.value_cache + blk + (long)lt * 16);
+            }
         }
     };
     // rows beyond the sequence's tokens (the tail of its last block) may hold anything: their K columns are masked
     // by the causal select, their V rows are cleared here so that 0 * garbage cannot reach the accumulators
     // j = block number within the item's range; it selects the LDS slots
-    auto stash = [&](KvRegs<U8>& r, int j) __attribute__((always_inline)) {
+    auto stash = [&](KvRegs<U8> (&rs)[UPT], int j) __attribute__((always_inline)) {
         const int tile = tile_at(j);
-        if (loader && j < cnt) {
-            const bool live = tile * TOK + ltid / CPR < kv_len;
-            uint8_t* kd = smem + kslot(j) * TILEK + lds_k;
-            uint8_t* vd = smem + vslot(j) * TILEV + lds_v;
+#pragma unroll
+        for (int uu = 0; uu < UPT; ++uu) {
+        KvRegs<U8>& r = rs[uu];
+        const int lt = unit_id(uu);
+        if (unit_loads(uu) && j < cnt) {
+            const bool live = tile * TOK + lt / CPR < kv_len;
+            uint8_t* kd = smem + kslot(j) * TILEK + unit_lds_k(uu);
+            uint8_t* vd = smem + vslot(j) * TILEV + unit_lds_v(uu);
             if constexpr (U8) {
                 // Codes go to LDS as 16-bit words holding (code - c) * 2^-24, c the integer nearest the row's
                 // zero-point: an exact f16 subnormal either way, but the sums the matrix pipe forms stay near the
@@ -382,8 +397,8 @@ void pa_prefill16_kernel(PrefillArgs a) {
                                                   centred(__builtin_amdgcn_perm(0u, v0, 0x0c030c02u), vneg),
                                                   centred(__builtin_amdgcn_perm(0u, v1, 0x0c010c00u), vneg),
                                                   centred(__builtin_amdgcn_perm(0u, v1, 0x0c030c02u), vneg)};
-                if (ltid % CPR == 0) {  // the table holds what is left of the zero-points
-                    float* hdr = reinterpret_cast<float*>(smem + OFF_H + (j & 3) * HDRB) + ltid / CPR;
+                if (lt % CPR == 0) {  // the table holds what is left of the zero-points
+                    float* hdr = reinterpret_cast<float*>(smem + OFF_H + (j & 3) * HDRB) + lt / CPR;
                     const float sck = __builtin_bit_cast(float, ksb);
                     hdr[0] = live ? sck : 0.0f;
                     hdr[TOK] = live ? (kzf - kc) * sck : 0.0f;
@@ -394,6 +409,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
                 *reinterpret_cast<u4v*>(kd) = r.k;
                 *reinterpret_cast<u4v*>(vd) = live ? r.v : u4v{0u, 0u, 0u, 0u};
             }
+        }
         }
     };
     const bool active = 16 * NG * wv < R;  // waves without rows only help moving blocks
@@ -722,12 +738,42 @@ void pa_prefill16_kernel(PrefillArgs a) {
         }
 #undef PA_DMA_STEP
         wait_vmem<0>();  // the clamped copies of the last three steps still target this workgroup's LDS
+    } else if constexpr (HALF) {
+        // Two register sets: block j + 2 goes from its set to LDS at the start of step j and the set takes block j + 4
+        // right behind it (the same two steps between a fetch and its use as with three sets, 16 registers fewer).
+        static_assert(!PIPE && !XATT, "dense items, a block worked through in one go");
+        fetch(set[0], 0);
+        fetch(set[1], 1);
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qreg[gi][s]));
+        stash(set[0], 0);
+        fetch(set[0], 2);
+        stash(set[1], 1);
+        fetch(set[1], 3);
+        __syncthreads();
+        if (active && cnt > 0) whole(0);
+        __syncthreads();
+        for (int j = 0; j < cnt; j += 2) {
+            stash(set[0], j + 2);
+            fetch(set[0], j + 4);
+            if (active && j + 1 < cnt) whole(j + 1);
+            __syncthreads();
+            if (j + 1 >= cnt) break;
+            stash(set[1], j + 3);
+            fetch(set[1], j + 5);
+            if (active && j + 2 < cnt) whole(j + 2);
+            __syncthreads();
+        }
     } else {
         fetch(set[0], 0);
         fetch(set[1], 1);
         fetch(set[2], 2);
         // step 0 multiplies V slot 3 by zero probabilities: make sure it holds numbers
-        if (loader) *reinterpret_cast<u4v*>(smem + 3 * TILEV + lds_v) = u4v{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int uu = 0; uu < UPT; ++uu)
+            if (unit_loads(uu)) *reinterpret_cast<u4v*>(smem + 3 * TILEV + unit_lds_v(uu)) = u4v{0u, 0u, 0u, 0u};
         // the query loads (issued above, tracked by the compiler) are waited for here, not inside the loop
     #pragma unroll
         for (int gi = 0; gi < NG; ++gi)
@@ -920,7 +966,7 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
     if (a.n_wide > 0) {  // items with more than 16 query rows
         PrefillArgs w = a;
         w.n_items = a.n_wide;
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, true, false, false>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(512), 0, s, w);
+        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, false, false, true>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(256), 0, s, w);
     }
     const int n_narrow = a.n_items - a.n_sparse - a.n_wide - (a.skip_single ? a.n_single : 0);
     if (n_narrow > 0) {  // the rest of the dense ones, listed behind them

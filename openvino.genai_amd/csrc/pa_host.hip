@@ -372,7 +372,7 @@ pa::XattDev xatt_dev(const pa_ctx* ctx) {
     return d;
 }
 
-// Work items of the MFMA kernel: tiles of QT query tokens (QT x G <= 256 rows) against ranges of KV blocks sized so
+// Work items of the MFMA kernel: tiles of QT query tokens (QT x G <= 128 rows) against ranges of KV blocks sized so
 // that the launch has several hundred workgroups of comparable length.  Listed as: items with more than 16 query
 // rows (u8 caches), the other dense ones, then the items of block-sparse sequences.
 void plan_items(pa_ctx* ctx) {
@@ -380,8 +380,9 @@ void plan_items(pa_ctx* ctx) {
     const int32_t* past = ctx->h_past.data();
     const int32_t* sb = ctx->h_sb.data();
     const int32_t G = ctx->cfg.num_heads / ctx->cfg.num_kv_heads;
-    // 16-bit caches: every dense item goes to the narrow kernel variant (128 query rows per workgroup, four waves per
-    // SIMD), which outruns the wide one there; u8 caches need the wide variant's registers
+    // 16-bit caches: every dense item goes to one kernel variant (16 rows per wave, four waves per SIMD; chunk-only
+    // launches to the straight-to-LDS variant).  u8 caches: items with more than 16 rows go to a variant of their own
+    // (32 rows per wave, two waves per SIMD) and are listed first
     const bool narrow_all = ctx->cfg.kv_cache_dtype != PA_U8;
     const int32_t QT = std::max(1, 128 / G), QTX = std::max(1, 128 / G), sw = ctx->sliding_window;
     struct Tile { int32_t b, q0, nq, lo, hi, kind; };  // kind 0: more than 16 rows, 1: the rest, 2: single-token sequences, 3: block-sparse

@@ -5,17 +5,16 @@
 //   logit = scale * sc_k * (q . codes - zp_k * sum(q))
 //   out   = sum_t w_t codes_t - sum_t w_t zp_v,   w_t = p_t * sc_v  (the same f16-rounded w_t on both sides)
 //
-// Work item = (sequence, tile of QT query tokens, range of KV blocks, kv head): one 512-thread
-// workgroup.  The query rows of the tile are the (token, head-in-group) pairs that share the kv head
-// -- up to 256 rows, 32 per wave in two 16-row groups -- so a KV block fetched once serves the whole
+// Work item = (sequence, tile of QT query tokens, range of KV blocks, kv head): one workgroup of 512
+// or 256 threads.  The query rows of the tile are the (token, head-in-group) pairs that share the kv head
+// -- up to 128 rows, 16 or 32 per wave -- so a KV block fetched once serves the whole
 // GQA group and QT tokens.  Long contexts are cut into ranges of KV blocks (split-K) so that work
 // items stay comparable in length; their partial (max, denominator, accumulator) rows are merged
 // by a second kernel.
-// KV blocks (32 tokens) travel global -> registers (three blocks in flight per thread) -> LDS (two K
-// slots, four V slots, one barrier per block); K rows are read back as MFMA A operands with
+// KV blocks (32 tokens) travel global -> registers (two or three blocks in flight per thread) -> LDS (two K
+// slots, four V slots, one barrier per block), or straight into LDS; K rows are read back as MFMA A operands with
 // ds_read_b128, V rows through the LDS transpose read (ds_read_b64_tr_b16), which hands each lane
-// four consecutive tokens of one channel.  The loop is software-pipelined over three blocks: QK of the
-// next block and PV of the previous one are issued around the softmax arithmetic of the current one.
+// four consecutive tokens of one channel.  A block is worked through in one go: QK, softmax, rescale, PV.
 //   S^T[token][row] = K . Q^T          v_mfma_f32_16x16x32_{f16,bf16}
 //   O^T[d][row]    += V^T . P^T        P (u8 caches: P times the V row's scale) in the operand type as hi + lo
 //                                      halves; one half alone (8 bits for bf16, 11 for f16) leaves outputs outside
@@ -156,13 +155,15 @@ __device__ __forceinline__ void wait_vmem() {
 
 // DT: type of the MFMA operands and of the rows staged in LDS; QDT: type of query and output; U8: the cache holds
 // `f32 scale | f32 zero-point | D codes` rows; codes go to LDS as 16-bit words, headers to a small table beside them.
-// NG: 16-row groups per wave.  2 = up to 256 query rows per workgroup; 1 = up to 128, the variant for work items
-// with few rows (single-token sequences: G rows), where the second group would only cost arithmetic.
-// PIPE: the three-block software pipeline described at the loop (needs the registers of two waves per SIMD);
-// without it a block is worked through in one go and the kernel fits four waves per SIMD (16-bit caches; the u8
-// path needs more registers and stays at two).
-// XATT: the work items belong to block-sparse sequences (never together with PIPE: passing over a block would have
-// to be threaded through three pipeline stages).
+// NG: 16-row groups per wave.  1 = up to 128 query rows per 512-thread workgroup, the variant for mixed steps over
+// 16-bit caches and for work items with few rows (single-token sequences: G rows), where a second group would only cost
+// arithmetic; it fits four waves per SIMD over 16-bit caches.  2 = 32 rows per wave (the 256-thread variants below).
+// A block is worked through in one go: QK, softmax, rescale, PV.
+// XATT: the work items belong to block-sparse sequences.
+// HALF: 256-thread workgroups of 128 rows whose KV blocks go through registers, two load units per thread (u8 caches,
+// whose codes are widened on the way to LDS): two such workgroups share a CU and fill in for each other at the
+// barriers.  (One 512-thread workgroup of 256 rows per CU, with a three-block software pipeline inside each wave, took
+// 0.296 ms for what this variant does in 0.255 ms: a third of the launch had neither pipe busy.)
 // DMA: 256-thread workgroups whose KV blocks go straight from global memory into LDS (four K and four V slots, three
 // blocks in flight behind the one being worked on).  Rows sit in LDS unpadded; instead the 16-byte pieces of a row are
 // permuted: K row r keeps piece p at position p ^ (r & 15) (16 lanes read one piece of 16 rows), V row r at
@@ -171,13 +172,13 @@ __device__ __forceinline__ void wait_vmem() {
 // that belongs at its LDS position.  With no
 // staging registers the kernel fits three waves per SIMD at two 16-row groups per wave: half the LDS operand traffic
 // per matrix instruction of the one-group variant.
-template <int D, int DT, int QDT, bool U8, int NG, bool PIPE, bool XATT, bool DMA, bool HALF = false>
-__global__ __launch_bounds__((DMA || HALF) ? 256 : 512, (DMA || HALF) ? 2 : (PIPE || U8) ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
+template <int D, int DT, int QDT, bool U8, int NG, bool XATT, bool DMA, bool HALF = false>
+__global__ __launch_bounds__((DMA || HALF) ? 256 : 512, (DMA || HALF) ? 2 : U8 ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
 void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
-    static_assert(!XATT || !PIPE, "the block-sparse variant works a block through in one go");
     static_assert(U8 || DT == QDT, "16-bit caches are used in the query's type");
-    static_assert(!DMA || (!U8 && !PIPE && !XATT && D == 128), "the straight-to-LDS variant: dense items, 16-bit caches, head size 128");
+    static_assert(!DMA || (!U8 && !XATT && D == 128), "the straight-to-LDS variant: dense items, 16-bit caches, head size 128");
+    static_assert(!(DMA && HALF) && (!HALF || (NG == 2 && !XATT)), "the register variant of 256 threads: dense items, two row groups per wave");
     constexpr int NT = (DMA || HALF) ? 256 : 512;
     constexpr int NCH = TOK * (D * 2 / 16);  // 16-byte chunks (eight codes of a u8 row) per block and tensor: 512 (D = 128) or 256 (D = 64)
     constexpr int UPT = HALF ? NCH / NT : 1;  // load units (a chunk, or eight codes and a row header) per thread and tensor
@@ -193,8 +194,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(DMA || NCH <= NT * UPT, "one chunk per load unit");
     constexpr int HDRB = U8 ? 4 * TOK * 4 : 0;  // per buffer: sc_k | zp_k * sc_k | sc_v | zp_v, one f32 per token each
     constexpr float CODE_UNIT = 16777216.0f;    // a code byte read as f16 is code * 2^-24
-    // The loop works on three blocks at once (see the pipeline below): K of block t+1, V of block t-1 and the
-    // headers of block t are read while block t+2 is written, hence two K slots and four V / header slots.
+    // Block t+1 is read while block t+2 is written: two K slots; the V and header slots are indexed modulo four.
     constexpr int OFF_V = NKS * TILEK, OFF_H = NKS * TILEK + NVS * TILEV;
     __shared__ __align__(16) uint8_t smem[DMA ? 16 : NKS * TILEK + NVS * TILEV + 4 * HDRB];  // K slots | V slots | headers[4]
     // DMA: every slot is an LDS object of its own, so that the compiler can tell a copy into one slot from the operand
@@ -480,10 +480,6 @@ void pa_prefill16_kernel(PrefillArgs a) {
             }
         }
     };
-    auto qk_pv = [&](bool do_qk, int jk, f4 (&sc)[2][2], bool do_pv, int jv, const u4v (&pb)[2], const u4v (&pl)[2])
-                     __attribute__((always_inline)) {
-        qk_pv_at(do_qk, smem + kslot(jk) * TILEK, sc, do_pv, smem + OFF_V + vslot(jv) * TILEV, pb, pl);
-    };
     // masks + online softmax of block `tile` (number j): probabilities as MFMA operands, rescale factors.
     // The running maximum is only raised when a block exceeds it by more than 2^4: probabilities then stay
     // below 16 and the accumulators are rescaled a few times per row instead of once per block.
@@ -598,52 +594,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
         }
     };
 
-    // ---- the pipeline -------------------------------------------------------------------------------------
-    // Step j (block t = tb + j) runs three independent pieces of work, so that the matrix pipe is busy while
-    // the vector pipe does the softmax:
-    //     S(t+1) = K(t+1) . Q^T          [MFMA]   K(t+1) was written to LDS during step j-1
-    //     O     += V(t-1)^T . P(t-1)^T   [MFMA]   P(t-1) was computed in step j-1
-    //     P(t)   = softmax step on S(t)  [VALU]   S(t) was computed in step j-1
-    // then rescales O by the factor block t produced, writes block t+2 to LDS and meets the other waves.
-    f4 s_cur[2][2];
-    u4v pb_prev[2], pl_prev[2];
-#pragma unroll
-    for (int gi = 0; gi < NG; ++gi) pb_prev[gi] = pl_prev[gi] = u4v{0u, 0u, 0u, 0u};
-    auto body = [&](auto masked_c, int j) __attribute__((always_inline)) {
-        f4 s_next[2][2];
-        u4v pb[2], pl[2];
-        float corr[2];
-        const bool all_kept[2] = {true, true};
-        qk_pv(true, j + 1, s_next, true, j + 3, pb_prev, pl_prev);  // blocks j + 1 and j - 1 (V slots are modulo 4)
-        softmax(masked_c, s_cur, tb + j, j, pb, pl, corr, all_kept);
-        // keep the softmax arithmetic in this block, next to the matrix instructions it overlaps with (its results
-        // are only consumed in the next step, and the compiler would otherwise sink it below the branches that follow)
-#pragma unroll
-        for (int gi = 0; gi < NG; ++gi) {
-            asm volatile("" : "+v"(pb[gi]), "+v"(corr[gi]), "+v"(l_part[gi]));
-            asm volatile("" : "+v"(pl[gi]));
-            if (U8) asm volatile("" : "+v"(zsum[gi]));
-        }
-        // issue order for the block above: the matrix instructions in program order, vector work in between
-#pragma unroll
-        for (int m = 0; m < NG * (2 * KS + RT * 2); ++m) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-        }
-#pragma unroll
-        for (int gi = 0; gi < NG; ++gi) {
-            if (__any(corr[gi] != 1.0f)) {
-#pragma unroll
-                for (int r = 0; r < RT; ++r) acc[gi][r] *= corr[gi];
-            }
-            pb_prev[gi] = pb[gi];
-            pl_prev[gi] = pl[gi];
-            s_cur[gi][0] = s_next[gi][0];
-            s_cur[gi][1] = s_next[gi][1];
-        }
-    };
-
-    // without the pipeline: block number j start to end (QK, softmax, rescale, PV)
+    // block number j start to end (QK, softmax, rescale, PV)
     auto body_whole = [&](auto masked_c, int j, const bool (&kept)[2], const uint8_t* kb, const uint8_t* vb)
                           __attribute__((always_inline)) {
         f4 sc[2][2];
@@ -741,7 +692,6 @@ void pa_prefill16_kernel(PrefillArgs a) {
     } else if constexpr (HALF) {
         // Two register sets: block j + 2 goes from its set to LDS at the start of step j and the set takes block j + 4
         // right behind it (the same two steps between a fetch and its use as with three sets, 16 registers fewer).
-        static_assert(!PIPE && !XATT, "dense items, a block worked through in one go");
         fetch(set[0], 0);
         fetch(set[1], 1);
 #pragma unroll
@@ -783,29 +733,16 @@ void pa_prefill16_kernel(PrefillArgs a) {
         fetch(set[0], 3);
         stash(set[1], 1);
         __syncthreads();
-        if (active) {
-            if (PIPE)
-                qk_pv(true, 0, s_cur, false, 0, pb_prev, pl_prev);
-            else if (cnt > 0)  // a block-sparse item may have nothing left to do
-                whole(0);
-        }
+        if (active && cnt > 0) whole(0);  // (a block-sparse item may have nothing left to do)
         __syncthreads();  // step 0 overwrites K slot 0, which the lines above read
-        // step j: set (j+1)%3 was written to LDS in step j-1 and takes block t+4; set (j+2)%3 holds block t+2.
-        // Without the pipeline step j works on block t+1 (whose K and V are both in LDS by then); block tb was done above.
+        // step j: set (j+1)%3 was written to LDS in step j-1 and takes block t+4; set (j+2)%3 holds block t+2; the
+        // step works on block t+1 (whose K and V are both in LDS by then); block tb was done above.
     #define PA_STEP(K)                                                                       \
         {                                                                                    \
-            const int j = i + K, tile = tb + j; /* PIPE is never block-sparse */           \
+            const int j = i + K;                                                             \
             if (j >= cnt) break;                                                             \
             fetch(set[(K + 1) % 3], j + 4);                                                  \
-            if (active) {                                                                    \
-                if (!PIPE) {                                                                 \
-                    if (j + 1 < cnt) whole(j + 1);                                           \
-                } else if (tile * TOK < free_lo || tile * TOK + TOK - 1 > free_hi) { /* wave-uniform */ \
-                    body(std::true_type{}, j);                                               \
-                } else {                                                                     \
-                    body(std::false_type{}, j);                                              \
-                }                                                                            \
-            }                                                                                \
+            if (active && j + 1 < cnt) whole(j + 1);                                         \
             stash(set[(K + 2) % 3], j + 2);                                                  \
             __syncthreads();                                                                 \
         }
@@ -816,7 +753,6 @@ void pa_prefill16_kernel(PrefillArgs a) {
         }
     #undef PA_STEP
     }
-    if (PIPE && active) qk_pv(false, 0, s_cur, true, te - 1 - tb, pb_prev, pl_prev);  // the last block's V
 
     // ---- write the rows ------------------------------------------------------------------------------
     const bool final_out = item.nsplit == 1;
@@ -963,10 +899,14 @@ __global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(PrefillArgs a) 
 template <int D, int DT, int QDT, bool U8>
 static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1) {
     if (ev0) (void)hipEventRecord(ev0, s);
-    if (a.n_wide > 0) {  // items with more than 16 query rows
-        PrefillArgs w = a;
-        w.n_items = a.n_wide;
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, false, false, true>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(256), 0, s, w);
+    if constexpr (U8) {
+        if (a.n_wide > 0) {  // u8 caches: the items with more than 16 query rows (up to 128) come first in the list
+            PrefillArgs w = a;
+            w.n_items = a.n_wide;
+            hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, false, true>), dim3((unsigned)w.n_items * a.sh.Hkv), dim3(256), 0, s, w);
+        }
+    } else if (a.n_wide > 0) {
+        return hipErrorInvalidValue;  // (16-bit caches list no such group)
     }
     const int n_narrow = a.n_items - a.n_sparse - a.n_wide - (a.skip_single ? a.n_single : 0);
     if (n_narrow > 0) {  // the rest of the dense ones, listed behind them
@@ -980,10 +920,10 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
         if constexpr (!U8 && D == 128) straight = a.n_single == 0 || a.skip_single;
         if constexpr (!U8 && D == 128) {
             if (straight)
-                hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, false, true>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(256), 0, s, nrw);
+                hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 2, false, true>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(256), 0, s, nrw);
         }
         if (!straight)
-            hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, false, false>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(512), 0, s, nrw);
+            hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, false>), dim3((unsigned)nrw.n_items * a.sh.Hkv), dim3(512), 0, s, nrw);
     }
     if (a.n_sparse > 0) {  // the items of block-sparse sequences come last
         PrefillArgs sp = a;
@@ -991,7 +931,7 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
         sp.n_items = a.n_sparse;
         // 128 query rows per workgroup whatever the cache: the fewer tokens share a work item, the fewer KV blocks
         // it has to walk for rows that did not keep them
-        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, false, true, false>), dim3((unsigned)sp.n_items * a.sh.Hkv), dim3(512), 0, s, sp);
+        hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, true, false>), dim3((unsigned)sp.n_items * a.sh.Hkv), dim3(512), 0, s, sp);
     }
     if (ev1) (void)hipEventRecord(ev1, s);
     if (a.n_merge > 0) {

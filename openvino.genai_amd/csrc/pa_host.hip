@@ -324,12 +324,46 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
             cap = std::min<int32_t>(most, (int32_t)(budget / (64 * G)));
             while (cap > 1 && !fits(cap)) --cap;
         }
+        *cap_out = cap;
+        if (waves == 4) {
+            // Four-wave workgroups, two to a CU: the count with the shortest estimated launch.  Measured on 32-token
+            // tiles of D = 128 (us): a workgroup alone on its CU takes t1 per tile; once workgroups share CUs (more than
+            // half the slots taken) the ones that share take f2 times as long and set the pace; all of them together
+            // cannot pull more than the memory system gives (5.8 TB/s in this access pattern); whole rounds of
+            // workgroups run one after the other and a last, partial round at the pace of its own occupancy; splits
+            // pay for the merge and score launch, which grows with the partial rows.  (Against the rule this replaces
+            // -- at least one round of workgroups, at least 16 blocks each, rounds 85 % full -- batches of 24 to 56
+            // sequences x 8 kv heads run 10 - 26 % faster, because they are not cut at all; full batches and long
+            // contexts come out the same within 2 %.)
+            const double t1 = (u8 ? 0.36 : 0.52) * c.head_size / 128.0, f2 = u8 ? 1.6 : 2.1;
+            const double tile_bytes = 2.0 * 32 * (u8 ? c.head_size + 8 : 2 * c.head_size), bw = 5.8e6;
+            auto t_tile = [&](int64_t w) {  // per tile, with w workgroups running at once
+                return std::max(w <= slots / 2 ? t1 : t1 * f2, (double)w * tile_bytes / bw);
+            };
+            int32_t best_n = 0;
+            double best_t = 0.0;
+            for (int32_t n = 1; n <= std::min(most, 64); ++n) {
+                const int32_t per = (most + n - 1) / n;
+                if (per > cap) continue;
+                const int64_t w = pairs * n, full = w / slots, rem = w % slots;
+                // (a cut that fills its rounds exactly is preferred over one that does not at equal estimates: the
+                // estimate of a partly filled round is the less certain one -- 8 x 32769 runs 2 % faster in 8 than in 7)
+                const double t = ((double)full * per * t_tile(slots) + (rem > 0 ? per * t_tile(rem) : 0.0)) *
+                                     (n > 1 && rem > 0 ? 1.02 : 1.0) +
+                                 (n > 1 ? 4.0 + 0.013 * (double)w : 0.0);
+                if (best_n == 0 || t < best_t) {
+                    best_n = n;
+                    best_t = t;
+                }
+            }
+            if (best_n > 0) return best_n;
+        }
+        // (eight-wave workgroups, one to a CU, and contexts that fit no count up to 64)
         int32_t s = 1;
         // aim for at least one round of workgroups, keep at least 16 blocks per workgroup (with fewer, what the
         // extra workgroups gain is lost again in the merge and score kernels)
         while (pairs * s < slots && most / (s + 1) >= 16) ++s;
         while ((most + s - 1) / s > cap) ++s;
-        *cap_out = cap;
         // more than one round of workgroups: a last round that is mostly empty costs a whole round's time; take
         // more splits until the rounds are at least 85 % full (sequences of one length, the worst case, in mind)
         auto fill = [&](int32_t n) {

@@ -326,19 +326,24 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
         }
         *cap_out = cap;
         if (waves == 4) {
-            // Four-wave workgroups, two to a CU: the count with the shortest estimated launch.  Measured on 32-token
-            // tiles of D = 128 (us): a workgroup alone on its CU takes t1 per tile; once workgroups share CUs (more than
-            // half the slots taken) the ones that share take f2 times as long and set the pace; all of them together
-            // cannot pull more than the memory system gives (5.8 TB/s in this access pattern); whole rounds of
-            // workgroups run one after the other and a last, partial round at the pace of its own occupancy; splits
-            // pay for the merge and score launch, which grows with the partial rows.  (Against the rule this replaces
-            // -- at least one round of workgroups, at least 16 blocks each, rounds 85 % full -- batches of 24 to 56
-            // sequences x 8 kv heads run 10 - 26 % faster, because they are not cut at all; full batches and long
-            // contexts come out the same within 2 %.)
-            const double t1 = (u8 ? 0.36 : 0.52) * c.head_size / 128.0, f2 = u8 ? 1.6 : 2.1;
-            const double tile_bytes = 2.0 * 32 * (u8 ? c.head_size + 8 : 2 * c.head_size), bw = 5.8e6;
+            // Four-wave workgroups, two to a CU: the count with the shortest estimated launch.  The estimate (us, per
+            // 32-token tile of D = 128; fitted to sweeps over batch sizes and contexts of 1024 - 12288 tokens with the
+            // count forced, 4 - 5 % rms): a workgroup alone on its CU takes t1 per tile; once workgroups share CUs (more
+            // than half the slots taken) the ones that share take t2 and set the pace; all of them together cannot pull
+            // more than the memory system gives in this access pattern (`bw`, less when probabilities are kept);
+            // whole rounds of workgroups run one after the other and a last, partial round at the pace of its own
+            // occupancy; splits pay for the merge and score launch, which grows with the partial rows.  (Against the
+            // rule this replaces -- at least one round of workgroups, at least 16 blocks each, rounds 85 % full --
+            // batches of 24 to 56 sequences x 8 kv heads run 10 - 26 % faster, because they are not cut at all; full
+            // batches and long contexts come out the same within 2 %.)
+            const bool sc = want_scores;
+            const double dscale = c.head_size / 128.0;
+            const double t1 = (u8 ? (sc ? 0.316 : 0.276) : (sc ? 0.495 : 0.478)) * dscale;
+            const double t2 = (u8 ? (sc ? 0.525 : 0.468) : (sc ? 1.104 : 1.064)) * dscale;
+            const double tile_bytes = 2.0 * 32 * (u8 ? c.head_size + 8 : 2 * c.head_size), bw = sc ? 5.9e6 : 6.97e6;
+            const double post_a = u8 ? (sc ? 2.4 : 1.0) : (sc ? 4.2 : 2.8), post_b = u8 ? (sc ? 0.0079 : 0.0066) : (sc ? 0.0050 : 0.0046);
             auto t_tile = [&](int64_t w) {  // per tile, with w workgroups running at once
-                return std::max(w <= slots / 2 ? t1 : t1 * f2, (double)w * tile_bytes / bw);
+                return std::max(w <= slots / 2 ? t1 : t2, (double)w * tile_bytes / bw);
             };
             int32_t best_n = 0;
             double best_t = 0.0;
@@ -350,7 +355,7 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
                 // estimate of a partly filled round is the less certain one -- 8 x 32769 runs 2 % faster in 8 than in 7)
                 const double t = ((double)full * per * t_tile(slots) + (rem > 0 ? per * t_tile(rem) : 0.0)) *
                                      (n > 1 && rem > 0 ? 1.02 : 1.0) +
-                                 (n > 1 ? 4.0 + 0.013 * (double)w : 0.0);
+                                 (n > 1 ? post_a + post_b * (double)w : 0.0);
                 if (best_n == 0 || t < best_t) {
                     best_n = n;
                     best_t = t;

@@ -454,8 +454,16 @@ void plan_items(pa_ctx* ctx) {
     // workgroups: cutting their short items further adds workgroups nobody waits for and a merge pass for their rows
     // (four 512-token prompts from scratch: 42.8 -> 33.6 us over bf16, 56.5 -> 44.4 us over u8; a single one, whose 116
     // to 128 workgroups leave most of the chip idle, is better off cut: 29.9 against 35.2 us over u8).
-    const int64_t shortest = (int64_t)tiles.size() * ctx->cfg.num_kv_heads >= 384 ? 16 : 8;
-    const int64_t target = std::min<int64_t>(128, std::max<int64_t>(shortest, total_blocks * ctx->cfg.num_kv_heads / 768));
+    const bool round_filled = (int64_t)tiles.size() * ctx->cfg.num_kv_heads >= 384;
+    const int64_t shortest = round_filled ? 16 : 8;
+    int64_t target = std::min<int64_t>(128, std::max<int64_t>(shortest, total_blocks * ctx->cfg.num_kv_heads / 768));
+    // ... and tiles of about one length that fill the round by themselves are not cut at all: there is nothing to
+    // balance (32 sequences x 64 tokens behind 500: 62.6 -> 42.6 us over bf16, 77.2 -> 56.1 us over u8)
+    if (round_filled && !tiles.empty()) {
+        int64_t longest = 0;
+        for (const Tile& t : tiles) longest = std::max<int64_t>(longest, t.hi - t.lo);
+        if (2 * longest * (int64_t)tiles.size() <= 3 * total_blocks) target = std::min<int64_t>(128, std::max(target, longest));
+    }
     // single-token sequences as items of the kernel variant that can hand their probabilities to the score kernel
     const bool stash_ok = narrow_all && G <= 16;
     ctx->stash_ok = stash_ok;

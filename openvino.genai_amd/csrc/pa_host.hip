@@ -56,6 +56,29 @@ struct DevBuf {
     T* as() const { return static_cast<T*>(p); }
 };
 
+// Pinned host memory that only ever grows (allocated, never registered): uploads from it are plain DMA, where a
+// pageable source of a few hundred KB is pinned and unpinned by the runtime on every copy.
+struct PinnedBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    void reserve(size_t bytes) {
+        if (bytes <= cap) return;
+        if (p) HIP_CHECK(hipHostFree(p));
+        p = nullptr;
+        cap = 0;
+        const size_t want = std::max<size_t>(bytes + bytes / 2, 4096);
+        HIP_CHECK(hipHostMalloc(&p, want, hipHostMallocDefault));
+        cap = want;
+    }
+    void release() {
+        if (p) (void)hipHostFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <class T>
+    T* as() const { return static_cast<T*>(p); }
+};
+
 void check_config(const pa_config* c) {
     PA_REQUIRE(c, PA_INVALID_C_PARAM, "config is null");
     PA_REQUIRE(c->num_heads > 0 && c->num_kv_heads > 0 && c->num_heads % c->num_kv_heads == 0, PA_PARAMETER_MISMATCH,
@@ -149,7 +172,7 @@ struct pa_ctx {
     // per-(sequence, split) descriptors of both plans
     struct DecPlan { int32_t nsplit = 1, max_tiles = 1, waves = 4; } dec_plan[2];
     size_t desc_off[2] = {0, 0};       // byte offsets of the two descriptor arrays in a table's buffer
-    std::vector<uint8_t> table_staging;
+    PinnedBuf table_staging;           // free again when a call returns: every upload from it is waited for
     bool shared_table = true;
     // workspace
     DevBuf part_acc, part_ml, final_ml, logits, group_scores, p_split, pf_part_acc, pf_part_ml;
@@ -249,6 +272,7 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
             const int32_t sub_shift = bs <= 32 ? 0 : __builtin_ctz((unsigned)(bs / 32));
             for (int32_t s = 0; s < nsplit; ++s) {
                 pa::DecodeDesc& d = out[i * nsplit + s];
+                std::memset(d.pad, 0, sizeof(d.pad));
                 d.b = b;
                 d.t = ctx->h_sb[b];
                 d.kv_len = kv_len;
@@ -858,6 +882,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->meta.release();
     ctx->items.release();
     for (auto& t : ctx->tables) t.release();
+    ctx->table_staging.release();
     ctx->part_acc.release();
     ctx->part_ml.release();
     ctx->final_ml.release();
@@ -1022,14 +1047,17 @@ int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int
                 ctx->desc_off[w] = total;
                 total += ctx->h_dec.size() * ctx->dec_plan[w].nsplit * sizeof(pa::DecodeDesc);
             }
-        std::vector<uint8_t>& stage = ctx->table_staging;
-        stage.assign(total, 0);
-        std::memcpy(stage.data(), ids, (size_t)count * sizeof(int32_t));
-        if (with_descs) fill_decode_descs(ctx, ids, stage.data());
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));
-        ctx->tables[idx].reserve(total);
-        HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, stage.data(), total, hipMemcpyHostToDevice, ctx->stream));
+        ctx->table_staging.reserve(total);
+        uint8_t* stage = ctx->table_staging.as<uint8_t>();
+        std::memcpy(stage, ids, (size_t)count * sizeof(int32_t));
+        std::memset(stage + (size_t)count * sizeof(int32_t), 0, std::max<size_t>(id_bytes, 128) - (size_t)count * sizeof(int32_t));
+        if (with_descs) fill_decode_descs(ctx, ids, stage);
+        if (ctx->tables[idx].cap < total) {  // kernels in flight may still read the buffer this would free
+            HIP_CHECK(hipStreamSynchronize(ctx->stream));
+            ctx->tables[idx].reserve(total);
+        }
+        HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, stage, total, hipMemcpyHostToDevice, ctx->stream));
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->table_count[idx] = count;
         ctx->table_bound[idx] = bound;

@@ -337,10 +337,170 @@ struct SingleScores {
     const int32_t* seq_list;
     int32_t n_seqs, gx;
 };
+// The matrix kernel's rows whose context was cut into several ranges: what folding their partials takes.  The fold
+// runs as a launch of its own or, when a score launch follows anyway, as extra workgroups of that launch (`n_wg` of
+// them, 16 rows each); the score rows then form the maximum and denominator of such a row from the partial ones
+// themselves instead of waiting for `final_ml`.  n_merge == 0: no such rows.
+struct MergeRows {
+    const float* part_acc;        // [T*Hq*max_split, D] un-normalised partial rows
+    const float* part_ml;         // [T*Hq*max_split, 2] (max in the log2 domain, denominator)
+    float* final_ml;              // [T*Hq, 2]
+    uint16_t* out;
+    const int32_t* merge_tokens;  // [n_merge]
+    const int32_t* tok_nsplit;    // [T]
+    const int32_t* single_idx;    // [B]
+    const int32_t* token_seq;     // [T]
+    int32_t n_merge, max_split, skip_single, Hq;
+    int32_t n_wg;                 // workgroups of 256 threads that fold the rows: ceil(n_merge * Hq / 16)
+};
+inline MergeRows merge_rows_of(const PrefillArgs& a) {
+    MergeRows m{};
+    m.part_acc = a.part_acc;
+    m.part_ml = a.part_ml;
+    m.final_ml = a.final_ml;
+    m.out = a.out;
+    m.merge_tokens = a.merge_tokens;
+    m.tok_nsplit = a.tok_nsplit;
+    m.single_idx = a.single_idx;
+    m.token_seq = a.st.token_seq;
+    m.n_merge = a.n_merge;
+    m.max_split = a.max_split;
+    m.skip_single = a.skip_single;
+    m.Hq = a.sh.Hq;
+    m.n_wg = (int32_t)(((long)a.n_merge * a.sh.Hq + 15) / 16);
+    return m;
+}
 #if defined(__HIPCC__)
+// Natural-log maximum and denominator of query row `rid` (token `tok`): from `final_ml`, or folded from the row's
+// partial ones when its context was cut into ranges that `m` describes.  (The fold is a call, not inline code: inside
+// the replay's row loop it would cost the kernel 16 registers.)
+__device__ inline __attribute__((noinline)) float2 fold_max_and_sum(const float2* pm, int ns) {
+    constexpr float LN2_ = 0.6931471805599453f;
+    float M = -INFINITY;
+    for (int s = 0; s < ns; ++s) M = fmaxf(M, pm[s].x);
+    float L = 0.0f;
+    for (int s = 0; s < ns; ++s) {
+        const float2 v = pm[s];
+        L += v.x == -INFINITY ? 0.0f : v.y * __builtin_amdgcn_exp2f(v.x - M);
+    }
+    return make_float2(M * LN2_, L);
+}
+// The same fold as inline code with four partial pairs in flight at a time (running maximum and rescaled sum), for
+// places with registers to spare: a round trip per four ranges instead of one per range.
+__device__ __forceinline__ float2 fold_max_and_sum_wide(const float2* pm, int ns) {
+    constexpr float LN2_ = 0.6931471805599453f;
+    float M = -INFINITY, L = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 4) {
+        float2 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = pm[min(s0 + j, ns - 1)];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j >= ns || v[j].x == -INFINITY) continue;
+            const float Mn = fmaxf(M, v[j].x);
+            L = L * __builtin_amdgcn_exp2f(M - Mn) + v[j].y * __builtin_amdgcn_exp2f(v[j].x - Mn);
+            M = Mn;
+        }
+    }
+    return make_float2(M * LN2_, L);
+}
+__device__ __forceinline__ float2 row_max_and_sum_wide(const float* __restrict__ final_ml, const MergeRows& m, int tok,
+                                                       long rid) {
+    const int ns = m.n_merge > 0 ? m.tok_nsplit[tok] : 1;
+    if (ns <= 1) return *reinterpret_cast<const float2*>(final_ml + 2 * rid);
+    return fold_max_and_sum_wide(reinterpret_cast<const float2*>(m.part_ml) + rid * m.max_split, ns);
+}
+__device__ __forceinline__ float2 row_max_and_sum(const float* __restrict__ final_ml, const MergeRows& m, int tok,
+                                                  long rid) {
+    const int ns = m.n_merge > 0 ? m.tok_nsplit[tok] : 1;
+    if (ns <= 1) return *reinterpret_cast<const float2*>(final_ml + 2 * rid);
+    return fold_max_and_sum(reinterpret_cast<const float2*>(m.part_ml) + rid * m.max_split, ns);
+}
+
+// Sixteen lanes per row, D / 16 channels each (16-byte loads), four rows per wave, workgroup `wg` of 256 threads;
+// ranges are folded in ascending order.  DT: type of the output rows.
+template <int D, int DT>
+__device__ __forceinline__ void merge_rows(const MergeRows& a, long wg) {
+    typedef float f4_ __attribute__((ext_vector_type(4)));
+    typedef uint32_t u4_ __attribute__((ext_vector_type(4)));
+    constexpr float LN2_ = 0.6931471805599453f;
+    constexpr int EPL = D / 16;
+    const int l16 = threadIdx.x & 15;
+    long idx = (wg * 256 + threadIdx.x) >> 4;
+    const long n_rows = (long)a.n_merge * a.Hq;
+    const bool live = idx < n_rows;
+    idx = min(idx, n_rows - 1);  // (surplus groups repeat the last row and store nothing: no divergence around the shuffles)
+    const int tok = a.merge_tokens[idx / a.Hq];
+    const long row = (long)tok * a.Hq + idx % a.Hq;
+    const bool mine = live && !(a.skip_single && a.single_idx[a.token_seq[tok]] >= 0);  // (else another kernel's row)
+    const int ns = a.tok_nsplit[tok];
+    float acc[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
+    float M, L;
+    if (ns <= 16) {
+        // lane s of the group holds range s: one round of loads instead of a dependent chain
+        const float2 ml = l16 < ns ? *reinterpret_cast<const float2*>(a.part_ml + 2 * (row * a.max_split + l16))
+                                   : make_float2(-INFINITY, 0.0f);
+        M = ml.x;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 16));
+        const float f_mine = ml.x == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml.x - M);
+        L = ml.y * f_mine;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) L += __shfl_xor(L, o, 16);
+        // four ranges per round, loaded unconditionally (indices clamped, surplus ones weighted zero) so that
+        // a round's loads are in flight together
+        for (int s0 = 0; s0 < ns; s0 += 4) {
+            float f[4];
+            f4_ v[4][EPL / 4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const long slot = row * a.max_split + min(s0 + j, ns - 1);
+                f[j] = __shfl(f_mine, min(s0 + j, ns - 1), 16);
+                if (s0 + j >= ns) f[j] = 0.0f;
+                const f4_* pa = reinterpret_cast<const f4_*>(a.part_acc + slot * D + l16 * EPL);
+#pragma unroll
+                for (int e = 0; e < EPL / 4; ++e) v[j][e] = pa[e];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < EPL; ++e)
+                    acc[e] = fmaf(f[j] == 0.0f ? 0.0f : v[j][e / 4][e % 4], f[j], acc[e]);  // fully masked ranges hold nothing
+        }
+    } else {
+        M = -INFINITY;
+        for (int s = 0; s < ns; ++s) M = fmaxf(M, a.part_ml[2 * (row * a.max_split + s)]);
+        L = 0.0f;
+        for (int s = 0; s < ns; ++s) {
+            const long slot = row * a.max_split + s;
+            const float ms = a.part_ml[2 * slot];
+            if (ms == -INFINITY) continue;
+            const float f = __builtin_amdgcn_exp2f(ms - M);
+            L += a.part_ml[2 * slot + 1] * f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + l16 * EPL + e] * f;
+        }
+    }
+    if (!mine) return;
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    uint32_t o[EPL / 2];
+#pragma unroll
+    for (int e = 0; e < EPL / 2; ++e)
+        o[e] = (uint32_t)store16<DT>(acc[2 * e] * inv) | ((uint32_t)store16<DT>(acc[2 * e + 1] * inv) << 16);
+    uint16_t* dst = a.out + row * D + l16 * EPL;
+    if constexpr (EPL == 8) *reinterpret_cast<u4_*>(dst) = u4_{o[0], o[1], o[2], o[3]};
+    else *reinterpret_cast<uint2*>(dst) = make_uint2(o[0], o[1]);
+    if (l16 == 0) {
+        a.final_ml[2 * row] = M * LN2_;
+        a.final_ml[2 * row + 1] = L;
+    }
+}
+
 __device__ __forceinline__ void single_scores_rows(const StepDev& st, const Shape& sh, const SingleScores& ss,
-                                                   const float* __restrict__ final_ml, float* __restrict__ scores,
-                                                   const int row, const int bx) {
+                                                   const float* __restrict__ final_ml, const MergeRows& mg,
+                                                   float* __restrict__ scores, const int row, const int bx) {
     __shared__ float s_ml[2 * 256];  // [Hq][2]: final maximum (log2 domain), 1 / denominator
     constexpr float LOG2E_ = 1.4426950408889634f;
     if (bx >= ss.gx) return;
@@ -353,7 +513,7 @@ __device__ __forceinline__ void single_scores_rows(const StepDev& st, const Shap
     float* out = scores + so;
     const int Hq = sh.Hq;
     for (int h = threadIdx.x; h < Hq; h += 256) {
-        const float2 ml = *reinterpret_cast<const float2*>(final_ml + 2 * ((long)t * Hq + h));
+        const float2 ml = row_max_and_sum_wide(final_ml, mg, t, (long)t * Hq + h);
         s_ml[2 * h] = ml.x * LOG2E_;
         s_ml[2 * h + 1] = ml.y > 0.0f ? 1.0f / ml.y : 0.0f;
     }
@@ -391,8 +551,9 @@ __device__ __forceinline__ void single_scores_rows(const StepDev& st, const Shap
     }
 }
 #endif
+// merge_later: the fold of the rows cut into ranges is left to the caller (`launch_scores_replay` takes it along).
 hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, int kv_dtype, hipEvent_t ev0,
-                            hipEvent_t ev1);
+                            hipEvent_t ev1, bool merge_later = false);
 
 // ---- block-sparse prefill (XAttention): the estimate's launch ---------------------------------
 struct XattTile {           // one workgroup-sized piece of the strided logits: 32 query groups x 128 key groups
@@ -430,11 +591,13 @@ hipError_t launch_rotate(hipStream_t s, void* key_cache, int kv_dtype, const Sha
                          const int32_t* rotated_block_indices, const int32_t* deltas, int32_t deltas_per_block,
                          int32_t n_rotated, const float* trig_lut);
 
-// Scores by replaying the last W query rows of every sequence against the positions they see (needs final_ml).
+// Scores by replaying the last W query rows of every sequence against the positions they see (needs final_ml, or
+// the partial maxima and denominators `mg` names for the rows cut into ranges; those rows' fold then runs as the last
+// workgroups of the same launch).
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
                                 float* final_ml, float* scores, int32_t max_kv_len, const int32_t* seq_list,
-                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss);
+                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss, const MergeRows& mg);
 
 // Block diversity of the evictable area (pa_rkv_diversity.hip).
 struct RkvDivSeq {          // one sequence whose diversity is computed

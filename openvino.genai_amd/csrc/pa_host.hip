@@ -818,24 +818,31 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
             a.tile_max = ctx->tile_max.as<float>();
         }
         if (!use_decode && !use_decode16) ctx->nsplit = ctx->max_split;
-        HIP_CHECK(pa::launch_prefill16(ctx->stream, a, c.query_dtype, c.kv_cache_dtype, ev0, ev1));
-        ctx->timed = ctx->profiling;
         // scores of the multi-token sequences (and of single-token ones that were work items of this kernel and kept
-        // nothing for the score rows): replay; the kept probabilities become scores in extra rows of the same launch
-        if (io->scores && !(use_decode16 && ctx->n_single == ctx->n_items)) {
-            pa::SingleScores ss{};
-            if (hand_over) {
-                ss.p_out = a.p_out;
-                ss.tile_max = a.tile_max;
-                ss.seq_list = ctx->dec16_list.as<int32_t>();
-                ss.n_seqs = (int32_t)ctx->h_dec16.size();
-            }
-            // (without the single-token sequences the launch has rows for the listed multi-token sequences only)
-            const bool singles_too = !(decode_u8_shape(c) || use_decode16 || hand_over);
+        // nothing for the score rows): replay; the kept probabilities become scores in extra rows of the same launch,
+        // and so does the fold of the rows that were cut into ranges (the score rows fold those rows' maxima and
+        // denominators themselves, so nothing in the launch waits for anything else in it)
+        const bool score_launch = io->scores && !(use_decode16 && ctx->n_single == ctx->n_items);
+        pa::SingleScores ss{};
+        if (score_launch && hand_over) {
+            ss.p_out = a.p_out;
+            ss.tile_max = a.tile_max;
+            ss.seq_list = ctx->dec16_list.as<int32_t>();
+            ss.n_seqs = (int32_t)ctx->h_dec16.size();
+        }
+        // (without the single-token sequences the launch has rows for the listed multi-token sequences only)
+        const bool singles_too = !(decode_u8_shape(c) || use_decode16 || hand_over);
+        const int32_t replay_seqs = singles_too ? ctx->B : (int32_t)ctx->h_multi.size();
+        const bool merge_later = score_launch && a.n_merge > 0 && replay_seqs + ss.n_seqs > 0 && ctx->max_kv > 0;
+        HIP_CHECK(pa::launch_prefill16(ctx->stream, a, c.query_dtype, c.kv_cache_dtype, ev0, ev1, merge_later));
+        ctx->timed = ctx->profiling;
+        if (score_launch) {
+            pa::MergeRows mg{};
+            if (merge_later) mg = pa::merge_rows_of(a);
             HIP_CHECK(pa::launch_scores_replay(ctx->stream, ctx->dev, a.sh, c.query_dtype, c.kv_cache_dtype, io->query,
                                                io->key_cache, table, a.final_ml, io->scores, ctx->max_kv,
-                                               singles_too ? nullptr : ctx->multi_list.as<int32_t>(),
-                                               singles_too ? ctx->B : (int32_t)ctx->h_multi.size(), a.xatt, ss));
+                                               singles_too ? nullptr : ctx->multi_list.as<int32_t>(), replay_seqs,
+                                               a.xatt, ss, mg));
         }
     }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)

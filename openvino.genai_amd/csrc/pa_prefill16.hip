@@ -816,88 +816,17 @@ void pa_prefill16_kernel(PrefillArgs a) {
     }
 }
 
-// Rows whose context was cut into several ranges: fold the partials (maxima in the log2 domain).  Sixteen lanes per
-// row, D / 16 channels each (16-byte loads), four rows per wave; ranges are folded in ascending order.
+// Rows whose context was cut into several ranges: fold the partials (maxima in the log2 domain).
 template <int D, int DT>
-__global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(PrefillArgs a) {
-    constexpr int EPL = D / 16;
-    const int l16 = threadIdx.x & 15;
-    long idx = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
-    const long n_rows = (long)a.n_merge * a.sh.Hq;
-    const bool live = idx < n_rows;
-    idx = min(idx, n_rows - 1);  // (surplus groups repeat the last row and store nothing: no divergence around the shuffles)
-    const int tok = a.merge_tokens[idx / a.sh.Hq];
-    const long row = (long)tok * a.sh.Hq + idx % a.sh.Hq;
-    const bool mine = live && !(a.skip_single && a.single_idx[a.st.token_seq[tok]] >= 0);  // (else another kernel's row)
-    const int ns = a.tok_nsplit[tok];
-    float acc[EPL];
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
-    float M, L;
-    if (ns <= 16) {
-        // lane s of the group holds range s: one round of loads instead of a dependent chain
-        const float2 ml = l16 < ns ? *reinterpret_cast<const float2*>(a.part_ml + 2 * (row * a.max_split + l16))
-                                   : make_float2(-INFINITY, 0.0f);
-        M = ml.x;
-#pragma unroll
-        for (int o = 8; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 16));
-        const float f_mine = ml.x == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml.x - M);
-        L = ml.y * f_mine;
-#pragma unroll
-        for (int o = 8; o > 0; o >>= 1) L += __shfl_xor(L, o, 16);
-        // four ranges per round, loaded unconditionally (indices clamped, surplus ones weighted zero) so that
-        // a round's loads are in flight together
-        for (int s0 = 0; s0 < ns; s0 += 4) {
-            float f[4];
-            f4 v[4][EPL / 4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const long slot = row * a.max_split + min(s0 + j, ns - 1);
-                f[j] = __shfl(f_mine, min(s0 + j, ns - 1), 16);
-                if (s0 + j >= ns) f[j] = 0.0f;
-                const f4* pa = reinterpret_cast<const f4*>(a.part_acc + slot * D + l16 * EPL);
-#pragma unroll
-                for (int e = 0; e < EPL / 4; ++e) v[j][e] = pa[e];
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int e = 0; e < EPL; ++e)
-                    acc[e] = fmaf(f[j] == 0.0f ? 0.0f : v[j][e / 4][e % 4], f[j], acc[e]);  // fully masked ranges hold nothing
-        }
-    } else {
-        M = -INFINITY;
-        for (int s = 0; s < ns; ++s) M = fmaxf(M, a.part_ml[2 * (row * a.max_split + s)]);
-        L = 0.0f;
-        for (int s = 0; s < ns; ++s) {
-            const long slot = row * a.max_split + s;
-            const float ms = a.part_ml[2 * slot];
-            if (ms == -INFINITY) continue;
-            const float f = __builtin_amdgcn_exp2f(ms - M);
-            L += a.part_ml[2 * slot + 1] * f;
-#pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + l16 * EPL + e] * f;
-        }
-    }
-    if (!mine) return;
-    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-    uint32_t o[EPL / 2];
-#pragma unroll
-    for (int e = 0; e < EPL / 2; ++e)
-        o[e] = (uint32_t)store16<DT>(acc[2 * e] * inv) | ((uint32_t)store16<DT>(acc[2 * e + 1] * inv) << 16);
-    uint16_t* dst = a.out + row * D + l16 * EPL;
-    if constexpr (EPL == 8) *reinterpret_cast<u4v*>(dst) = u4v{o[0], o[1], o[2], o[3]};
-    else *reinterpret_cast<uint2*>(dst) = make_uint2(o[0], o[1]);
-    if (l16 == 0) {
-        a.final_ml[2 * row] = M * LN2;
-        a.final_ml[2 * row + 1] = L;
-    }
+__global__ __launch_bounds__(256) void pa_prefill16_merge_kernel(MergeRows m) {
+    merge_rows<D, DT>(m, blockIdx.x);
 }
 
 }  // namespace
 
 template <int D, int DT, int QDT, bool U8>
-static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1) {
+static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1,
+                                         bool merge_later) {
     if (ev0) (void)hipEventRecord(ev0, s);
     if constexpr (U8) {
         if (a.n_wide > 0) {  // u8 caches: the items with more than 16 query rows (up to 128) come first in the list
@@ -934,29 +863,29 @@ static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hi
         hipLaunchKernelGGL((pa_prefill16_kernel<D, DT, QDT, U8, 1, true, false>), dim3((unsigned)sp.n_items * a.sh.Hkv), dim3(512), 0, s, sp);
     }
     if (ev1) (void)hipEventRecord(ev1, s);
-    if (a.n_merge > 0) {
-        const long rows = (long)a.n_merge * a.sh.Hq;
-        hipLaunchKernelGGL((pa_prefill16_merge_kernel<D, QDT>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
+    if (a.n_merge > 0 && !merge_later) {
+        const MergeRows m = merge_rows_of(a);
+        hipLaunchKernelGGL((pa_prefill16_merge_kernel<D, QDT>), dim3((unsigned)m.n_wg), dim3(256), 0, s, m);
     }
     return hipGetLastError();
 }
 
 template <int D>
 static hipError_t launch_prefill16_d(hipStream_t s, const PrefillArgs& a, int q_dtype, int kv_dtype, hipEvent_t ev0,
-                                     hipEvent_t ev1) {
+                                     hipEvent_t ev1, bool merge_later) {
     if (kv_dtype == DT_U8)
-        return q_dtype == DT_F16 ? launch_prefill16_typed<D, DT_F16, DT_F16, true>(s, a, ev0, ev1)
-                                 : launch_prefill16_typed<D, DT_F16, DT_BF16, true>(s, a, ev0, ev1);
+        return q_dtype == DT_F16 ? launch_prefill16_typed<D, DT_F16, DT_F16, true>(s, a, ev0, ev1, merge_later)
+                                 : launch_prefill16_typed<D, DT_F16, DT_BF16, true>(s, a, ev0, ev1, merge_later);
     if (kv_dtype != q_dtype) return hipErrorInvalidValue;
-    return q_dtype == DT_F16 ? launch_prefill16_typed<D, DT_F16, DT_F16, false>(s, a, ev0, ev1)
-                             : launch_prefill16_typed<D, DT_BF16, DT_BF16, false>(s, a, ev0, ev1);
+    return q_dtype == DT_F16 ? launch_prefill16_typed<D, DT_F16, DT_F16, false>(s, a, ev0, ev1, merge_later)
+                             : launch_prefill16_typed<D, DT_BF16, DT_BF16, false>(s, a, ev0, ev1, merge_later);
 }
 
 hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, int kv_dtype, hipEvent_t ev0,
-                            hipEvent_t ev1) {
+                            hipEvent_t ev1, bool merge_later) {
     if (a.n_items == 0) return hipSuccess;
-    if (a.sh.D == 128) return launch_prefill16_d<128>(s, a, q_dtype, kv_dtype, ev0, ev1);
-    if (a.sh.D == 64) return launch_prefill16_d<64>(s, a, q_dtype, kv_dtype, ev0, ev1);
+    if (a.sh.D == 128) return launch_prefill16_d<128>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
+    if (a.sh.D == 64) return launch_prefill16_d<64>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     return hipErrorInvalidValue;
 }
 

@@ -58,13 +58,18 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
                                                              const float* __restrict__ final_ml,
                                                              float* __restrict__ scores,
                                                              const int32_t* __restrict__ seq_list, int n_seqs,
-                                                             XattDev xd, SingleScores ss) {
+                                                             XattDev xd, SingleScores ss, MergeRows mg) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     constexpr int KS = D / 32;
     constexpr int CROWB = U8 ? D + 8 : D * 2;
     constexpr float CODE_UNIT = 16777216.0f;  // a code byte read as f16 is code * 2^-24
+    if ((int)blockIdx.y >= n_seqs + ss.n_seqs) {  // the last rows: the fold of the matrix kernel's partial rows
+        const long wg = (long)((int)blockIdx.y - n_seqs - ss.n_seqs) * gridDim.x + blockIdx.x;
+        if (wg < mg.n_wg) merge_rows<D, QDT>(mg, wg);
+        return;
+    }
     if ((int)blockIdx.y >= n_seqs) {  // the rows behind the sequences': single-token sequences whose probabilities were kept
-        single_scores_rows(st, sh, ss, final_ml, scores, (int)blockIdx.y - n_seqs, (int)blockIdx.x);
+        single_scores_rows(st, sh, ss, final_ml, mg, scores, (int)blockIdx.y - n_seqs, (int)blockIdx.x);
         return;
     }
     const int b = seq_list ? seq_list[blockIdx.y] : (int)blockIdx.y;  // the listed sequences, or all of the step's
@@ -88,6 +93,12 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
     const float scl = st.scale * LOG2E;
     const float inv_g = 1.0f / (float)G;
     const int xi = xd.seq_of ? xd.seq_of[b] : -1;  // block-sparse sequence: the wave's 32 positions lie in one key block
+
+    // Rows cut into ranges, one query token, at most 64 heads (the usual case): lane h folds head h's maximum and
+    // denominator once, up front, and the row loop below fetches them from that lane.
+    const bool lane_rows = mg.n_merge > 0 && W == 1 && Hq <= WAVE;
+    float2 ml_lane = make_float2(0.0f, 0.0f);
+    if (lane_rows) ml_lane = row_max_and_sum_wide(final_ml, mg, first_tok, (long)first_tok * Hq + min(lane, Hq - 1));
 
     float total[CG];
 #pragma unroll
@@ -159,7 +170,13 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
                     const int row = min(r0 + 4 * g + i, R - 1);
                     const int tok = (int)(((float)row + 0.5f) * inv_g);
                     const long rid = (long)(first_tok + tok) * Hq + hkv * G + (row - tok * G);
-                    const float2 ml = *reinterpret_cast<const float2*>(final_ml + 2 * rid);
+                    float2 ml;
+                    if (lane_rows) {
+                        const int head = hkv * G + (row - tok * G);
+                        ml = make_float2(__shfl(ml_lane.x, head, WAVE), __shfl(ml_lane.y, head, WAVE));
+                    } else {
+                        ml = row_max_and_sum(final_ml, mg, first_tok + tok, rid);
+                    }
                     m2[i] = ml.x * LOG2E;
                     inv_l[i] = ml.y > 0.0f ? 1.0f / ml.y : 0.0f;
                     rpos[i] = ok ? first_pos + tok : -1;  // -1: sees nothing
@@ -204,19 +221,23 @@ __global__ __launch_bounds__(256) void pa_scores_mfma_kernel(StepDev st, Shape s
 hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
                                 const void* query, const void* key_cache, const int32_t* block_indices,
                                 float* final_ml, float* scores, int32_t max_kv_len, const int32_t* seq_list,
-                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss_in) {
+                                int32_t n_seqs, const XattDev& xd, const SingleScores& ss_in, const MergeRows& mg_in) {
     SingleScores ss = ss_in;
     if (!ss.p_out) ss.n_seqs = 0;
-    if (n_seqs + ss.n_seqs == 0 || max_kv_len <= 0) return hipSuccess;
-    if (sh.Hq > 256 || n_seqs + ss.n_seqs > 65535) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)ceil_div(max_kv_len, 4 * TN), (unsigned)(n_seqs + ss.n_seqs)), block(256);
+    MergeRows mg = mg_in;
+    if (mg.n_merge <= 0) mg.n_wg = 0;
+    if (max_kv_len <= 0 || (n_seqs + ss.n_seqs == 0 && mg.n_wg == 0)) return mg.n_wg ? hipErrorInvalidValue : hipSuccess;
+    const int gx_all = ceil_div(max_kv_len, 4 * TN);
+    const int merge_rows_y = ceil_div(mg.n_wg, gx_all);
+    if (sh.Hq > 256 || n_seqs + ss.n_seqs + merge_rows_y > 65535) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)gx_all, (unsigned)(n_seqs + ss.n_seqs + merge_rows_y)), block(256);
     ss.gx = min(ceil_div(max_kv_len, 2048), 64);  // (at most the grid's width: 2048 > 4 * TN)
     auto q = reinterpret_cast<const uint16_t*>(query);
     auto k = reinterpret_cast<const uint8_t*>(key_cache);
 #define PA_REPLAY(DD, DT, Q, U8)                                                                               \
     {                                                                                                          \
         hipLaunchKernelGGL((pa_scores_mfma_kernel<DD, DT, Q, U8>), grid, block, 0, s, st, sh, q, k,            \
-                           block_indices, final_ml, scores, seq_list, n_seqs, xd, ss);                         \
+                           block_indices, final_ml, scores, seq_list, n_seqs, xd, ss, mg);                     \
         return hipGetLastError();                                                                              \
     }
     if (sh.bs < 16 || sh.bs > 256 || (sh.bs & (sh.bs - 1))) return hipErrorInvalidValue;

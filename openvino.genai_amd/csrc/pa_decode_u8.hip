@@ -495,15 +495,22 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     }
 }
 
-// Folds split partials (log2 domain) into the output row and the final (max, denominator).
+// Rows a launch's merge has to fold: every (token, head) of a step of single-token sequences, or those of the listed
+// sequences of a mixed step.
+__host__ __device__ inline long decode_merge_rows(const DecodeArgs& a) {
+    return (long)(a.seq_list ? a.n_seqs : a.st.T) * a.sh.Hq;
+}
+
+// Folds split partials (log2 domain) into the output row and the final (max, denominator); `r` counts the launch's rows.
 // WRITE_FAC: leave exp2(m_split - M) / L in place of the split denominators (for a score kernel that runs afterwards).
 template <int D, int QDT, bool WRITE_FAC>
-__device__ __forceinline__ void merge_row(const DecodeArgs& a, const long row, const int lane) {
+__device__ __forceinline__ void merge_row(const DecodeArgs& a, const long r, const int lane) {
     constexpr int EPL = D / 64;
-    if (row >= (long)a.st.T * a.sh.Hq) return;
-    if (a.seq_list) {  // mixed step: rows of multi-token sequences belong to another kernel
-        const int b = a.st.token_seq[row / a.sh.Hq];
-        if (a.st.subsequence_begins[b + 1] - a.st.subsequence_begins[b] != 1) return;
+    if (r >= decode_merge_rows(a)) return;
+    long row = r;
+    if (a.seq_list) {  // mixed step: the rows of the listed single-token sequences (the others are another kernel's)
+        const int i = (int)(r / a.sh.Hq);
+        row = (long)a.st.subsequence_begins[a.seq_list[i]] * a.sh.Hq + (r - (long)i * a.sh.Hq);
     }
     float M, inv, L;
     float acc[EPL];
@@ -706,7 +713,7 @@ hipError_t launch_decode_scores(hipStream_t s, const DecodeArgs& a, float* score
 }
 
 hipError_t launch_decode_merge(hipStream_t s, const DecodeArgs& a, int q_dtype) {
-    const dim3 grid((unsigned)(((long)a.st.T * a.sh.Hq + 3) / 4));
+    const dim3 grid((unsigned)((decode_merge_rows(a) + 3) / 4));
     if (a.sh.D == 128) {
         if (q_dtype == DT_F16) hipLaunchKernelGGL((pa_decode_merge_kernel<128, DT_F16>), grid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((pa_decode_merge_kernel<128, DT_BF16>), grid, dim3(256), 0, s, a);
@@ -722,7 +729,7 @@ hipError_t launch_decode_merge(hipStream_t s, const DecodeArgs& a, int q_dtype) 
 template <int D, int QDT>
 static hipError_t launch_post_typed(hipStream_t s, const DecodeArgs& a, float* scores, int max_kv_len) {
     const int gx = min(ceil_div(max_kv_len, 2048), 64);
-    const int merge_blocks = (int)(((long)a.st.T * a.sh.Hq + 3) / 4);
+    const int merge_blocks = (int)((decode_merge_rows(a) + 3) / 4);
     const size_t lds = (size_t)a.sh.Hq * a.nsplit * sizeof(float);
     hipLaunchKernelGGL((pa_decode_post_kernel<D, QDT>), dim3((unsigned)(merge_blocks + gx * a.n_seqs)), dim3(256), lds, s, a,
                        scores, merge_blocks, gx);

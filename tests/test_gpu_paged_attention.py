@@ -178,6 +178,11 @@ def test_decode_u8_kernel_shapes(pkg, dev, name, args, kw):
     ("pf16_f16_interleaved_items_window", (8, 2, 64, 32, "f16", "f16",
                                            [300] + [700 + 11 * i for i in range(9)], [50] + [1] * 9),
      {"sliding_window": 600, "score_aggregation_window": [5] + [1] * 9}),
+    # more than 64 query heads, contexts cut into several ranges: the score rows fold the ranges' maxima and
+    # denominators row by row (a wave's lanes hold at most 64 heads' pairs)
+    ("pf16_bf16_128_heads_ranges", (128, 8, 128, 32, "bf16", "bf16", [1500, 2000, 40], [300, 1, 1]), {}),
+    ("pf16_f16_96_heads_ranges_window_rows", (96, 8, 128, 32, "f16", "f16", [1200, 900], [200, 1]),
+     {"score_aggregation_window": [5, 1]}),
 ])
 def test_prefill16_kernel_shapes(pkg, dev, name, args, kw):
     _check(pkg, dev, H.case_from_lens(name, *args, **kw), 41)
@@ -192,6 +197,7 @@ def test_prefill16_kernel_shapes(pkg, dev, name, args, kw):
     ("pf_u8_prefill_only_long", (8, 2, 128, 32, "f16", "u8", [1500], [700]), {"score_aggregation_window": [16]}),
     ("pf_u8_g32_all_on_matrix_kernel", (32, 1, 128, 32, "f16", "u8", [64, 0, 300], [9, 8, 1]), {}),
     ("pf_u8_decode_multi_split_beside_prefill", (8, 2, 128, 32, "f16", "u8", [3000, 0, 2500], [1, 40, 1]), {}),
+    ("pf_u8_96_heads_ranges", (96, 8, 128, 32, "f16", "u8", [1200, 2500, 60], [200, 1, 1]), {}),
 ])
 def test_prefill_u8_kernel_shapes(pkg, dev, name, args, kw):
     got, ref, c = _check(pkg, dev, H.case_from_lens(name, *args, **kw), 43, outliers=True)

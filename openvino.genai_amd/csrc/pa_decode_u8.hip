@@ -643,7 +643,7 @@ __global__ __launch_bounds__(256) void pa_decode_scores_kernel(DecodeArgs a, flo
 template <int D, int QDT>
 __global__ __launch_bounds__(256) void pa_decode_post_kernel(DecodeArgs a, float* __restrict__ scores, int merge_blocks,
                                                              int gx) {
-    extern __shared__ float s_fac[];  // [Hq][nsplit]
+    extern __shared__ float s_fac[];  // [Hq][nsplit] factors, then [Hq][nsplit] (maximum, denominator) pairs
     const int id = blockIdx.x;
     if (id < merge_blocks) {
         merge_row<D, QDT, false>(a, (long)id * 4 + (threadIdx.x >> 6), threadIdx.x & 63);
@@ -652,15 +652,30 @@ __global__ __launch_bounds__(256) void pa_decode_post_kernel(DecodeArgs a, float
     const int sid = id - merge_blocks, bx = sid % gx, by = sid / gx;
     const int b = a.seq_list ? a.seq_list[by] : by;
     const int t = a.st.subsequence_begins[b];
+    // the sequence's (maximum, denominator) pairs, one per (head, split): every thread fetches its share with all
+    // loads in flight, then one thread per head folds its row out of LDS (a thread per head reading its row from
+    // global memory walked a chain of dependent loads: 3.5 us more on a step of one sequence)
+    const int n_pairs = a.sh.Hq * a.nsplit;
+    float2* s_ml = reinterpret_cast<float2*>(s_fac + n_pairs);  // [Hq][nsplit]
+    const float2* ml_g = reinterpret_cast<const float2*>(a.part_ml) + (long)t * n_pairs;
+    for (int i0 = threadIdx.x; i0 < n_pairs; i0 += 4 * 256) {
+        float2 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = ml_g[min(i0 + 256 * j, n_pairs - 1)];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + 256 * j < n_pairs) s_ml[i0 + 256 * j] = v[j];
+    }
+    __syncthreads();
     for (int h = threadIdx.x; h < a.sh.Hq; h += 256) {
-        const float* ml = a.part_ml + 2 * ((long)t * a.sh.Hq + h) * a.nsplit;
+        const float2* ml = s_ml + h * a.nsplit;
         float M = -INFINITY, L = 0.0f;
-        for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, ml[2 * s]);
+        for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, ml[s].x);
         for (int s = 0; s < a.nsplit; ++s)
-            if (ml[2 * s] != -INFINITY) L += ml[2 * s + 1] * __builtin_amdgcn_exp2f(ml[2 * s] - M);
+            if (ml[s].x != -INFINITY) L += ml[s].y * __builtin_amdgcn_exp2f(ml[s].x - M);
         const float inv = L > 0.0f ? 1.0f / L : 0.0f;
         for (int s = 0; s < a.nsplit; ++s)
-            s_fac[h * a.nsplit + s] = ml[2 * s] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[2 * s] - M) * inv;
+            s_fac[h * a.nsplit + s] = ml[s].x == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[s].x - M) * inv;
     }
     __syncthreads();
     score_positions<true>(a, scores, bx, gx, by, s_fac);
@@ -730,7 +745,7 @@ template <int D, int QDT>
 static hipError_t launch_post_typed(hipStream_t s, const DecodeArgs& a, float* scores, int max_kv_len) {
     const int gx = min(ceil_div(max_kv_len, 2048), 64);
     const int merge_blocks = (int)((decode_merge_rows(a) + 3) / 4);
-    const size_t lds = (size_t)a.sh.Hq * a.nsplit * sizeof(float);
+    const size_t lds = (size_t)a.sh.Hq * a.nsplit * 3 * sizeof(float);
     hipLaunchKernelGGL((pa_decode_post_kernel<D, QDT>), dim3((unsigned)(merge_blocks + gx * a.n_seqs)), dim3(256), lds, s, a,
                        scores, merge_blocks, gx);
     return hipGetLastError();

@@ -132,9 +132,28 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
     const int last_block = (kv_len + bsz - 1) / bsz - 1;  // a last tile of one 16-token block repeats it (rows masked)
     Block ba, bb;
     int tile = tb + wv;
+    // The step's new K / V row of this (sequence, kv head) goes into the caches here when the step's append is fused
+    // into this launch: by the wave that later reads the sequence's last tile, which waits for the two stores before
+    // it fetches that tile (at once when it is the wave's first tile, else in front of the fetch, see `process`).
+    const bool owner = a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
+    auto append_row = [&]() __attribute__((always_inline)) {
+        if (lane < 2 * CPR) {  // lanes 0 .. CPR-1: the K row's 16-byte pieces, the next CPR lanes: the V row's
+            const bool isv = lane >= CPR;
+            const int piece = isv ? lane - CPR : lane, pos = kv_len - 1;
+            const u4v row = *reinterpret_cast<const u4v*>(reinterpret_cast<const uint8_t*>(isv ? a.value : a.key) +
+                                                          ((long)t * Hkv + hkv) * ROWB + piece * 16);
+            const long dst = (((long)table[pos / bsz] * Hkv + hkv) * bsz + pos % bsz) * ROWB + piece * 16;
+            *reinterpret_cast<u4v*>(const_cast<uint8_t*>(isv ? a.value_cache : a.key_cache) + dst) = row;
+        }
+    };
+    if (owner && tile == tile_hi - 1) {
+        append_row();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     if (tile < te)
         issue(ba, table[min((BPT * tile) >> sub_shift, last_block)], table[min((BPT * tile + BPT - 1) >> sub_shift, last_block)],
               tile & sub_mask);
+    if (owner && tile != tile_hi - 1) append_row();
     for (int i = tid; i < BPT * (te - tb); i += 64 * WAVES) tab[i] = table[min((BPT * tb + i) >> sub_shift, last_block)];
 
     // query operand (B of QK): lane (n, g) holds q[head n][32 s + 8 g + e]; heads beyond the group are zero
@@ -156,6 +175,7 @@ __global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
 
     auto process = [&](Block& cur, Block& nxt, const int tl) __attribute__((always_inline)) {
         // next block's loads into flight, this block's V into the slot
+        if (owner && tl + WAVES == tile_hi - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the appended row is in place
         if (tl + WAVES < te) issue(nxt, tab[BPT * (tl + WAVES - tb)], tab[BPT * (tl + WAVES - tb) + BPT - 1], (tl + WAVES) & sub_mask);
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {

@@ -206,8 +206,8 @@ struct DecodeArgs {
     const int32_t* block_indices;
     const int32_t* seq_list;      // sequences this launch covers (single-token ones); null = all B
     const DecodeDesc* descs;      // u8 kernel: [n_seqs][nsplit]
-    const uint16_t* key;          // u8 kernel with fuse_append: the step's new K / V rows [T, Hkv*D], which the
-    const uint16_t* value;        // workgroup that owns a sequence's last block quantises into the caches itself
+    const uint16_t* key;          // with fuse_append: the step's new K / V rows [T, Hkv*D], which the workgroup that
+    const uint16_t* value;        // owns a sequence's last block writes (u8: quantises) into the caches itself
     int32_t fuse_append;
     int32_t n_seqs;
     int32_t G;                    // query heads per kv head (<= 16)

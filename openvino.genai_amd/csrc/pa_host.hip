@@ -666,8 +666,8 @@ DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_sc
     return w;
 }
 
-// fuse_append: the call is the attention half of pa_forward in a step whose sequences all go to the u8 decode kernel,
-// and no append kernel has run: the decode kernel writes the step's K / V rows itself.
+// fuse_append: the call is the attention half of pa_forward in a step whose sequences all go to one decode kernel (the
+// u8 one or the 16-bit one), and no append kernel has run: the decode kernel writes the step's K / V rows itself.
 void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static_ws = false, bool fuse_append = false) {
     check_io(ctx, layer, io, false, true);
     const int32_t* table = table_for(ctx, layer);
@@ -730,6 +730,9 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.total_scores = ctx->total_scores;
         plan_decode_u8(ctx, io->scores != nullptr, &a.nsplit, &a.max_tiles, &ctx->h_dec16);
         a.waves = 4;
+        a.key = static_cast<const uint16_t*>(io->key);
+        a.value = static_cast<const uint16_t*>(io->value);
+        a.fuse_append = fuse_append ? 1 : 0;
         a.n_seqs = (int32_t)ctx->h_dec16.size();
         a.seq_list = ctx->dec16_in_order ? nullptr : ctx->dec16_list.as<int32_t>();
         ctx->nsplit = a.nsplit;
@@ -1252,8 +1255,11 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
     if (!ctx) return PA_INVALID_C_PARAM;
     return guarded(ctx, [&] {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
-        // a step of single-token sequences over a u8 cache: the decode kernel appends the new rows itself
-        const bool fuse = ctx->step_ready && decode_u8_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B;
+        // a step of single-token sequences that all go to one of the decode kernels: it appends the new rows itself
+        const bool fuse = ctx->step_ready &&
+                          ((decode_u8_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B) ||
+                           (mfma_shape(ctx->cfg) && decode16_shape(ctx->cfg) && (int32_t)ctx->h_dec16.size() == ctx->B &&
+                            ctx->n_sparse == 0 && ctx->n_single == ctx->n_items));
         if (fuse) check_io(ctx, layer, io, true, false);
         else do_kv_append(ctx, layer, io);
         do_attention(ctx, layer, io, false, fuse);

@@ -124,7 +124,7 @@ typedef struct pa_layer_io {
 
 /* One layer's PagedAttention: KV append (+ u8 quantisation), attention, optional scores.  The op's `alibi_slopes`
  * input has no counterpart: no ALiBi term is applied, and a binding must refuse a non-empty slopes tensor.  Tuned
- * kernels serve block_size 16, 32, 64, 128 and 256, head size 64 / 128; other shapes run on a generic kernel.  In a step whose sequences all schedule one token over a u8 cache the append
+ * kernels serve block_size 16, 32, 64, 128 and 256, head size 64 / 128; other shapes run on a generic kernel.  In a step whose sequences all schedule one token (u8 cache, or an f16 / bf16 cache of the query's type) the append
  * is done by the attention kernel itself (the cache rows are the ones pa_kv_append writes). */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The two halves of pa_forward on their own (same arguments; pa_kv_append ignores query/out/scores,

@@ -325,10 +325,12 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
     const pa_config& c = ctx->cfg;
     const int32_t G = c.num_heads / c.num_kv_heads;
     int32_t most = 1;
+    int64_t all_tiles = 0;
     for (int32_t b : seqs ? *seqs : ctx->h_dec) {
         const int32_t kv = ctx->h_past[b] + 1;
         const int32_t first = ctx->sliding_window > 0 ? std::max(0, kv - ctx->sliding_window) : 0;
         most = std::max(most, (kv + 31) / 32 - first / 32);
+        all_tiles += (kv + 31) / 32 - first / 32;
     }
     const bool u8 = c.kv_cache_dtype == PA_U8;
     const int64_t pairs = (int64_t)(seqs ? seqs->size() : ctx->h_dec.size()) * c.num_kv_heads;
@@ -369,12 +371,18 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
             auto t_tile = [&](int64_t w) {  // per tile, with w workgroups running at once
                 return std::max(w <= slots / 2 ? t1 : t2, (double)w * tile_bytes / bw);
             };
+            // Contexts of unequal length: every sequence is cut into the same number of parts, so its workgroups are
+            // as much shorter than the longest one's as its context is; the launch then behaves like one of fewer
+            // workgroups of the longest kind (16 sequences x 64 - 2048 positions, D = 64: 6 parts instead of 3, the step
+            // 17.2 -> 16.4 us, 12.5 -> 11.2 us without scores; equal contexts are not touched).
+            const double fill = (double)all_tiles / ((double)most * (double)(pairs / c.num_kv_heads));
             int32_t best_n = 0;
             double best_t = 0.0;
             for (int32_t n = 1; n <= std::min(most, 64); ++n) {
                 const int32_t per = (most + n - 1) / n;
                 if (per > cap) continue;
-                const int64_t w = pairs * n, full = w / slots, rem = w % slots;
+                const int64_t w = pairs * n, w_run = std::max<int64_t>(1, std::llround((double)w * fill));
+                const int64_t full = w_run / slots, rem = w_run % slots;
                 // (a cut that fills its rounds exactly is preferred over one that does not at equal estimates: the
                 // estimate of a partly filled round is the less certain one -- 8 x 32769 runs 2 % faster in 8 than in 7)
                 const double t = ((double)full * per * t_tile(slots) + (rem > 0 ? per * t_tile(rem) : 0.0)) *

@@ -173,6 +173,10 @@ struct pa_ctx {
     struct DecPlan { int32_t nsplit = 1, max_tiles = 1, waves = 4; } dec_plan[2];
     size_t desc_off[2] = {0, 0};       // byte offsets of the two descriptor arrays in a table's buffer
     PinnedBuf table_staging;           // free again when a call returns: every upload from it is waited for
+    // the step's small arrays (packed metadata, work items, lists) pass through this pinned area on their way to the
+    // device: pieces are handed out front to back and are free again after the next wait for the stream
+    PinnedBuf step_staging;
+    size_t step_staged = 0;
     bool shared_table = true;
     // workspace
     DevBuf part_acc, part_ml, final_ml, logits, group_scores, p_split, pf_part_acc, pf_part_ml;
@@ -446,6 +450,23 @@ pa::XattDev xatt_dev(const pa_ctx* ctx) {
 // Work items of the MFMA kernel: tiles of QT query tokens (QT x G <= 128 rows) against ranges of KV blocks sized so
 // that the launch has several hundred workgroups of comparable length.  Listed as: items with more than 16 query
 // rows (u8 caches), the other dense ones, then the items of block-sparse sequences.
+// Queues a copy of `bytes` of host memory to `dst` on the context's stream, through the pinned staging area (from a
+// pageable source the runtime stages and waits per call, 15 - 20 us per array).  The caller waits for the stream before
+// it returns; with the area used up, the copies so far are waited for here and the area starts over (larger if needed).
+void stage_upload(pa_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return;
+    const size_t need = (bytes + 63) & ~(size_t)63;
+    if (ctx->step_staged + need > ctx->step_staging.cap) {
+        HIP_CHECK(hipStreamSynchronize(ctx->stream));
+        ctx->step_staged = 0;
+        ctx->step_staging.reserve(std::max<size_t>({need, (size_t)1 << 16, 2 * ctx->step_staging.cap}));
+    }
+    uint8_t* at = ctx->step_staging.as<uint8_t>() + ctx->step_staged;
+    std::memcpy(at, src, bytes);
+    ctx->step_staged += need;
+    HIP_CHECK(hipMemcpyAsync(dst, at, bytes, hipMemcpyHostToDevice, ctx->stream));
+}
+
 void plan_items(pa_ctx* ctx) {
     const int32_t B = ctx->B, T = ctx->T;
     const int32_t* past = ctx->h_past.data();
@@ -592,9 +613,8 @@ void plan_items(pa_ctx* ctx) {
     ctx->single_idx_off = item_bytes + (size_t)T * sizeof(int32_t);
     ctx->merge_tok_off = ctx->single_idx_off + (size_t)B * sizeof(int32_t);
     ctx->items.reserve(item_bytes + tok_ns.size() * sizeof(int32_t));
-    HIP_CHECK(hipMemcpyAsync(ctx->items.p, items.data(), item_bytes, hipMemcpyHostToDevice, ctx->stream));
-    HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(ctx->items.p) + item_bytes, tok_ns.data(),
-                             tok_ns.size() * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    stage_upload(ctx, ctx->items.p, items.data(), item_bytes);
+    stage_upload(ctx, static_cast<uint8_t*>(ctx->items.p) + item_bytes, tok_ns.data(), tok_ns.size() * sizeof(int32_t));
     // the sequences a score replay has rows for: those with more than one token, longest context first
     ctx->h_multi.clear();
     for (int32_t b = 0; b < B; ++b)
@@ -603,20 +623,18 @@ void plan_items(pa_ctx* ctx) {
                      [&](int32_t x, int32_t y) { return past[x] + sb[x + 1] - sb[x] > past[y] + sb[y + 1] - sb[y]; });
     if (!ctx->h_multi.empty()) {
         ctx->multi_list.reserve(ctx->h_multi.size() * sizeof(int32_t));
-        HIP_CHECK(hipMemcpyAsync(ctx->multi_list.p, ctx->h_multi.data(), ctx->h_multi.size() * sizeof(int32_t),
-                                 hipMemcpyHostToDevice, ctx->stream));
+        stage_upload(ctx, ctx->multi_list.p, ctx->h_multi.data(), ctx->h_multi.size() * sizeof(int32_t));
     }
     if (!ctx->h_dec16.empty()) {
         ctx->dec16_list.reserve(ctx->h_dec16.size() * sizeof(int32_t));
-        HIP_CHECK(hipMemcpyAsync(ctx->dec16_list.p, ctx->h_dec16.data(), ctx->h_dec16.size() * sizeof(int32_t),
-                                 hipMemcpyHostToDevice, ctx->stream));
+        stage_upload(ctx, ctx->dec16_list.p, ctx->h_dec16.data(), ctx->h_dec16.size() * sizeof(int32_t));
     }
     if (!ctx->h_dec.empty()) {
         ctx->dec_list.reserve(ctx->h_dec.size() * sizeof(int32_t));
-        HIP_CHECK(hipMemcpyAsync(ctx->dec_list.p, ctx->h_dec.data(), ctx->h_dec.size() * sizeof(int32_t),
-                                 hipMemcpyHostToDevice, ctx->stream));
+        stage_upload(ctx, ctx->dec_list.p, ctx->h_dec.data(), ctx->h_dec.size() * sizeof(int32_t));
     }
     HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    ctx->step_staged = 0;
     ctx->tok_nsplit_off = item_bytes;
     if (split_off_decode && !ctx->h_dec.empty())
         for (int w = 0; w < 2; ++w)
@@ -901,6 +919,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->items.release();
     for (auto& t : ctx->tables) t.release();
     ctx->table_staging.release();
+    ctx->step_staging.release();
     ctx->part_acc.release();
     ctx->part_ml.release();
     ctx->final_ml.release();
@@ -988,8 +1007,8 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         // the previous step's kernels may still read the old copy
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->meta.reserve(h.size() * sizeof(int32_t));
-        HIP_CHECK(hipMemcpyAsync(ctx->meta.p, h.data(), h.size() * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // `h` is pageable and leaves scope
+        ctx->step_staged = 0;
+        stage_upload(ctx, ctx->meta.p, h.data(), h.size() * sizeof(int32_t));  // (waited for at the end of plan_items)
 
         int32_t* d = ctx->meta.as<int32_t>();
         ctx->dev.past_lens = d;

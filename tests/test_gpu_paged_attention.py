@@ -84,6 +84,30 @@ def test_kv_append_many_rows_bit_exact(pkg, dev, qd, kd, D, Hkv, bs):
     assert np.array_equal(vc.cpu().numpy(), vc_ref), "value cache bytes differ"
 
 
+def test_step_arrays_outgrow_the_pinned_staging_area(pkg, dev):
+    """A context's step arrays pass through a pinned staging area that starts small: a step of 40000 tokens does not
+    fit it (the area is waited for and grows in the middle of the step's uploads), and the steps before and after it
+    on the same context use what is there."""
+    import torch
+    from oracle import oracle as O
+    Hkv, D, bs, qd, kd = 2, 64, 32, "f16", "u8"
+    op = pkg.PagedAttention(Hkv, Hkv, D, bs, qd, kd, 1, 0, torch.cuda.current_stream(dev))
+    for i, (past, new) in enumerate([([5, 0], [3, 40]), ([0, 31, 100], [25000, 14000, 1000]), ([7], [9])]):
+        c = H.build_case(H.case_from_lens(f"staging_{i}", Hkv, Hkv, D, bs, qd, kd, past, new), 90 + i)
+        kc_ref, vc_ref = c["key_cache0"].copy(), c["value_cache0"].copy()
+        O.kv_append(c["key"], c["value"], H.DT[qd], kc_ref, vc_ref, H.DT[kd], c["past_lens"], c["subsequence_begins"],
+                    c["block_indices"], c["block_indices_begins"], Hkv, D, bs)
+        k, v = H.to_device_16(torch, c["key"], qd, dev), H.to_device_16(torch, c["value"], qd, dev)
+        kc, vc = torch.from_numpy(c["key_cache0"]).to(dev), torch.from_numpy(c["value_cache0"]).to(dev)
+        op.step_begin(c["past_lens"], c["subsequence_begins"], c["block_indices_begins"],
+                      int((c["past_lens"] + c["new_lens"]).max()))
+        op.set_block_indices(c["block_indices"], c["num_blocks"])
+        op.kv_append(k, v, kc, vc)
+        op.synchronize()
+        assert np.array_equal(kc.cpu().numpy(), kc_ref), f"step {i}: key cache bytes differ"
+        assert np.array_equal(vc.cpu().numpy(), vc_ref), f"step {i}: value cache bytes differ"
+
+
 def test_kv_append_constant_and_extreme_rows(pkg, dev):
     # constant rows (zero range), huge range, and exact .5 ties
     import torch

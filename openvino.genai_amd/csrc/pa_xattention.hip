@@ -349,35 +349,37 @@ __global__ __launch_bounds__(256) void xatt_select_kernel(XattArgs a) {
     const int ncand = max(I - 1, 0);  // candidates J = 1 .. I - 1
     long long mine = 0;
     for (int J = tid; J <= I; J += 256) mine += fx[J];
-    part[tid] = mine;
     for (int J = 1 + tid; J < I; J += 256) {
         const float my = v[J];
         int rank = 0;
         for (int o = 1; o < I; ++o) rank += (v[o] > my || (v[o] == my && o < J)) ? 1 : 0;
         order[rank] = J;
     }
-    __syncthreads();
-    for (int step = 128; step > 0; step >>= 1) {
-        if (tid < step) part[tid] += part[tid + step];
-        __syncthreads();
-    }
-    const long long total_fx = part[0];
+    // the total: every wave adds its lanes' shares with lane swaps, the four wave sums meet in LDS (integers: the
+    // same total in any order)
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, WAVE);
+    if (lane == 0) part[wv] = mine;
+    __syncthreads();  // (also: `order` is complete)
+    const long long total_fx = part[0] + part[1] + part[2] + part[3];
     const long long forced = fx[0] + (I > 0 ? fx[I] : 0);
     const double required = (double)xs.threshold * (double)total_fx;
-    __syncthreads();
-    // prefix sums over the ranked candidates: thread t owns ranks [t * per, (t + 1) * per)
+    // prefix sums over the ranked candidates: thread t owns ranks [t * per, (t + 1) * per); inclusive scan inside the
+    // wave by lane shifts, the waves in front add their totals
     const int per = (ncand + 255) / 256;
     long long local = 0;
     for (int k = tid * per; k < min((tid + 1) * per, ncand); ++k) local += fx[order[k]];
-    part[tid] = local;
-    __syncthreads();
-    for (int step = 1; step < 256; step <<= 1) {  // inclusive scan of the 256 partials
-        const long long add = tid >= step ? part[tid - step] : 0;
-        __syncthreads();
-        part[tid] += add;
-        __syncthreads();
+    long long incl = local;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const long long up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
     }
-    long long kept = forced + (tid > 0 ? part[tid - 1] : 0);
+    if (lane == WAVE - 1) part[4 + wv] = incl;
+    __syncthreads();
+    long long before = incl - local;  // the ranks in front of this thread's
+    for (int w = 0; w < wv; ++w) before += part[4 + w];
+    long long kept = forced + before;
     uint32_t* out = a.mask + xs.mask_off + ((long)hq * xs.nqb + ib) * xs.words;
     for (int k = tid * per; k < min((tid + 1) * per, ncand); ++k) {
         if (!((double)kept < required)) break;

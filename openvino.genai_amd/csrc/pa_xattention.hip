@@ -276,24 +276,22 @@ __global__ __launch_bounds__(256) void xatt_select_kernel(XattArgs a) {
     for (int ig = i_lo + wv; ig < i_hi; ig += 4) {
         const float* row = logits + (long)(ig - xs.qs0) * xs.ld;
         float m = -INFINITY, l = 0.0f;
-        // eight values per lane and round, loaded before any is used (one load per round would leave the wave waiting
-        // for memory once per 64 values)
-        for (int j0 = 4 * lane; j0 <= ig; j0 += 512) {
-            const f4 xa = *reinterpret_cast<const f4*>(row + j0);
-            const f4 xb = *reinterpret_cast<const f4*>(row + min(j0 + 256, xs.ld - 4));
-            float x[8];
+        // twenty values per lane and round, loaded before any is used (a round is a trip to memory that the next one
+        // waits for: a row of up to 1280 strided keys takes one)
+        for (int j0 = 4 * lane; j0 <= ig; j0 += 1280) {
+            f4 xv[5];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                x[c] = j0 + c <= ig ? xa[c] : -INFINITY;
-                x[4 + c] = j0 + 256 + c <= ig ? xb[c] : -INFINITY;
-            }
+            for (int c = 0; c < 5; ++c) xv[c] = *reinterpret_cast<const f4*>(row + min(j0 + 256 * c, xs.ld - 4));
+            float x[20];
+#pragma unroll
+            for (int c = 0; c < 20; ++c) x[c] = j0 + 256 * (c >> 2) + (c & 3) <= ig ? xv[c >> 2][c & 3] : -INFINITY;
             float mx = x[0];
 #pragma unroll
-            for (int c = 1; c < 8; ++c) mx = fmaxf(mx, x[c]);
+            for (int c = 1; c < 20; ++c) mx = fmaxf(mx, x[c]);
             const float mn = fmaxf(m, mx);  // finite: x[0] is a visible value
             float add = 0.0f;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) add += __builtin_amdgcn_exp2f(x[c] - mn);
+            for (int c = 0; c < 20; ++c) add += __builtin_amdgcn_exp2f(x[c] - mn);
             l = l * __builtin_amdgcn_exp2f(m - mn) + add;
             m = mn;
         }

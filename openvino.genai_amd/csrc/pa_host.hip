@@ -172,9 +172,9 @@ struct pa_ctx {
     // per-(sequence, split) descriptors of both plans
     struct DecPlan { int32_t nsplit = 1, max_tiles = 1, waves = 4; } dec_plan[2];
     size_t desc_off[2] = {0, 0};       // byte offsets of the two descriptor arrays in a table's buffer
-    PinnedBuf table_staging;           // free again when a call returns: every upload from it is waited for
-    // the step's small arrays (packed metadata, work items, lists) pass through this pinned area on their way to the
-    // device: pieces are handed out front to back and are free again after the next wait for the stream
+    // the step's host arrays (packed metadata, work items, lists, block tables with their descriptors) pass through
+    // this pinned area on their way to the device: pieces are handed out front to back, their copies are queued and not
+    // waited for, and pa_step_begin starts over at the front once it has waited for the stream
     PinnedBuf step_staging;
     size_t step_staged = 0;
     bool shared_table = true;
@@ -450,20 +450,27 @@ pa::XattDev xatt_dev(const pa_ctx* ctx) {
 // Work items of the MFMA kernel: tiles of QT query tokens (QT x G <= 128 rows) against ranges of KV blocks sized so
 // that the launch has several hundred workgroups of comparable length.  Listed as: items with more than 16 query
 // rows (u8 caches), the other dense ones, then the items of block-sparse sequences.
-// Queues a copy of `bytes` of host memory to `dst` on the context's stream, through the pinned staging area (from a
-// pageable source the runtime stages and waits per call, 15 - 20 us per array).  The caller waits for the stream before
-// it returns; with the area used up, the copies so far are waited for here and the area starts over (larger if needed).
-void stage_upload(pa_ctx* ctx, void* dst, const void* src, size_t bytes) {
-    if (bytes == 0) return;
-    const size_t need = (bytes + 63) & ~(size_t)63;
+// A piece of the pinned staging area for an upload of `bytes` that the caller fills and queues on the context's stream.
+// With the area used up, the copies queued so far are waited for here and the area starts over (larger: it grows
+// until a whole step's pieces fit).
+uint8_t* stage_piece(pa_ctx* ctx, size_t bytes) {
+    const size_t need = (std::max<size_t>(bytes, 1) + 63) & ~(size_t)63;
     if (ctx->step_staged + need > ctx->step_staging.cap) {
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->step_staged = 0;
         ctx->step_staging.reserve(std::max<size_t>({need, (size_t)1 << 16, 2 * ctx->step_staging.cap}));
     }
     uint8_t* at = ctx->step_staging.as<uint8_t>() + ctx->step_staged;
-    std::memcpy(at, src, bytes);
     ctx->step_staged += need;
+    return at;
+}
+
+// Queues a copy of `bytes` of host memory to `dst` on the context's stream through the staging area (from a pageable
+// source the runtime stages and waits per call, 15 - 20 us per array); `src` is free when this returns.
+void stage_upload(pa_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return;
+    uint8_t* at = stage_piece(ctx, bytes);
+    std::memcpy(at, src, bytes);
     HIP_CHECK(hipMemcpyAsync(dst, at, bytes, hipMemcpyHostToDevice, ctx->stream));
 }
 
@@ -633,8 +640,6 @@ void plan_items(pa_ctx* ctx) {
         ctx->dec_list.reserve(ctx->h_dec.size() * sizeof(int32_t));
         stage_upload(ctx, ctx->dec_list.p, ctx->h_dec.data(), ctx->h_dec.size() * sizeof(int32_t));
     }
-    HIP_CHECK(hipStreamSynchronize(ctx->stream));
-    ctx->step_staged = 0;
     ctx->tok_nsplit_off = item_bytes;
     if (split_off_decode && !ctx->h_dec.empty())
         for (int w = 0; w < 2; ++w)
@@ -918,7 +923,6 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->meta.release();
     ctx->items.release();
     for (auto& t : ctx->tables) t.release();
-    ctx->table_staging.release();
     ctx->step_staging.release();
     ctx->part_acc.release();
     ctx->part_ml.release();
@@ -1008,7 +1012,7 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->meta.reserve(h.size() * sizeof(int32_t));
         ctx->step_staged = 0;
-        stage_upload(ctx, ctx->meta.p, h.data(), h.size() * sizeof(int32_t));  // (waited for at the end of plan_items)
+        stage_upload(ctx, ctx->meta.p, h.data(), h.size() * sizeof(int32_t));
 
         int32_t* d = ctx->meta.as<int32_t>();
         ctx->dev.past_lens = d;
@@ -1085,17 +1089,15 @@ int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int
                 total += ctx->h_dec.size() * ctx->dec_plan[w].nsplit * sizeof(pa::DecodeDesc);
             }
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
-        ctx->table_staging.reserve(total);
-        uint8_t* stage = ctx->table_staging.as<uint8_t>();
-        std::memcpy(stage, ids, (size_t)count * sizeof(int32_t));
-        std::memset(stage + (size_t)count * sizeof(int32_t), 0, std::max<size_t>(id_bytes, 128) - (size_t)count * sizeof(int32_t));
-        if (with_descs) fill_decode_descs(ctx, ids, stage);
         if (ctx->tables[idx].cap < total) {  // kernels in flight may still read the buffer this would free
             HIP_CHECK(hipStreamSynchronize(ctx->stream));
             ctx->tables[idx].reserve(total);
         }
+        uint8_t* stage = stage_piece(ctx, total);
+        std::memcpy(stage, ids, (size_t)count * sizeof(int32_t));
+        std::memset(stage + (size_t)count * sizeof(int32_t), 0, std::max<size_t>(id_bytes, 128) - (size_t)count * sizeof(int32_t));
+        if (with_descs) fill_decode_descs(ctx, ids, stage);
         HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, stage, total, hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->table_count[idx] = count;
         ctx->table_bound[idx] = bound;
     });

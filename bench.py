@@ -283,7 +283,7 @@ def diversity_leg(torch, op, spec, kc, dev, ev, reps=20):
 
 def rotation_leg(torch, pkg, op, spec, kc, dev, reps=10):
     """Cache rotation of every block of the workload's sequences (one layer, one delta per block): wall time of
-    the whole call (argument checks, one upload of the block list and deltas, two stream waits, one kernel),
+    the whole call (argument checks, the block list and deltas copied to pinned staging and queued, one kernel),
     events on the launch stream.  Rotates a copy of the K cache, in place."""
     Hkv, D, bs = spec["Hkv"], spec["D"], spec["bs"]
     blocks = np.ascontiguousarray(spec["block_indices"], np.int32)

@@ -40,7 +40,10 @@ struct DevBuf {
     size_t cap = 0;
     void reserve(size_t bytes) {
         if (bytes <= cap) return;
-        if (p) HIP_CHECK(hipFree(p));
+        if (p) {  // work in flight may still use the old buffer
+            HIP_CHECK(hipDeviceSynchronize());
+            HIP_CHECK(hipFree(p));
+        }
         p = nullptr;
         cap = 0;
         size_t want = std::max<size_t>(bytes, 256);
@@ -452,13 +455,13 @@ pa::XattDev xatt_dev(const pa_ctx* ctx) {
 // rows (u8 caches), the other dense ones, then the items of block-sparse sequences.
 // A piece of the pinned staging area for an upload of `bytes` that the caller fills and queues on the context's stream.
 // With the area used up, the copies queued so far are waited for here and the area starts over (larger: it grows
-// until a whole step's pieces fit).
+// until a whole step's pieces fit, up to 32 MiB -- beyond that a step pays such a wait now and then).
 uint8_t* stage_piece(pa_ctx* ctx, size_t bytes) {
     const size_t need = (std::max<size_t>(bytes, 1) + 63) & ~(size_t)63;
     if (ctx->step_staged + need > ctx->step_staging.cap) {
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
         ctx->step_staged = 0;
-        ctx->step_staging.reserve(std::max<size_t>({need, (size_t)1 << 16, 2 * ctx->step_staging.cap}));
+        ctx->step_staging.reserve(std::max<size_t>({need, (size_t)1 << 16, std::min<size_t>(2 * ctx->step_staging.cap, (size_t)32 << 20)}));
     }
     uint8_t* at = ctx->step_staging.as<uint8_t>() + ctx->step_staged;
     ctx->step_staged += need;
@@ -1433,13 +1436,13 @@ int32_t pa_rotate_cache(pa_ctx* ctx, void* key_cache, int64_t num_blocks, const 
             PA_REQUIRE(rotation_deltas[i] >= 0 && rotation_deltas[i] < ctx->trig_rows, PA_OUT_OF_BOUNDS,
                        "rotation delta beyond the trig table");
         HIP_CHECK(hipSetDevice(c.device));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // the previous call's kernel may still read the arguments
+        // (the previous call's kernel may still read the arguments: the copies below are ordered behind it on the
+        // stream, and a buffer that has to grow is freed by a call that waits for the device)
         ctx->rot_args.reserve((num_rotated + n_delta) * sizeof(int32_t));
         int32_t* d_idx = ctx->rot_args.as<int32_t>();
         int32_t* d_delta = d_idx + num_rotated;
-        HIP_CHECK(hipMemcpyAsync(d_idx, rotated_block_indices, num_rotated * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipMemcpyAsync(d_delta, rotation_deltas, n_delta * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // host arrays are the caller's, pageable
+        stage_upload(ctx, d_idx, rotated_block_indices, num_rotated * sizeof(int32_t));
+        stage_upload(ctx, d_delta, rotation_deltas, n_delta * sizeof(int32_t));
         HIP_CHECK(pa::launch_rotate(ctx->stream, key_cache, c.kv_cache_dtype, shape_of(c), d_idx, d_delta,
                                     deltas_per_block, num_rotated, ctx->trig_lut.as<float>()));
     });
@@ -1491,15 +1494,14 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         PA_REQUIRE(num_blocks >= ctx->table_bound[tidx] && num_blocks > 0, PA_OUT_OF_BOUNDS,
                    "the key cache holds fewer blocks than the block table of this layer refers to");
         HIP_CHECK(hipSetDevice(c.device));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // the previous call's kernels may still read the sequence list
+        // (the previous call's kernels may still read the sequence list and the work buffers: this call's copy and
+        // kernels are ordered behind them on the stream, and a buffer that has to grow is freed by a call that waits)
         const int chunks = pa::rkv_diversity_chunks(ev_max);
         ctx->div_seqs.reserve(seqs.size() * sizeof(pa::RkvDivSeq));
         ctx->div_stats.reserve((size_t)c.num_kv_heads * tok_total * sizeof(float4));
         ctx->div_mean.reserve((size_t)c.num_kv_heads * tok_total * sizeof(float));
         ctx->div_colsum.reserve(seqs.size() * c.num_kv_heads * (chunks + 1) * c.head_size * sizeof(float));
-        HIP_CHECK(hipMemcpyAsync(ctx->div_seqs.p, seqs.data(), seqs.size() * sizeof(pa::RkvDivSeq), hipMemcpyHostToDevice,
-                                 ctx->stream));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // `seqs` is pageable and leaves scope
+        stage_upload(ctx, ctx->div_seqs.p, seqs.data(), seqs.size() * sizeof(pa::RkvDivSeq));
         pa::RkvDivArgs a{};
         a.key_cache = static_cast<const uint8_t*>(key_cache);
         a.block_indices = ctx->tables[tidx].as<int32_t>();

@@ -1177,18 +1177,15 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
         }
         PA_REQUIRE(logit_off * 4 <= ((int64_t)4 << 30), PA_NOT_ALLOCATED,
                    "block-sparse prefill: the strided logits of this step exceed 4 GiB (larger stride or shorter chunks)");
-        // the previous step's kernels may still read the old plan
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));
+        // (pa_step_begin has waited for the previous step's kernels, which read the old plan; the copies are queued)
         const size_t seq_bytes = seqs.size() * sizeof(pa::XattSeq), tile_bytes = tiles.size() * sizeof(pa::XattTile);
         ctx->x_tiles_off = seq_bytes;
         ctx->x_seq_of_off = seq_bytes + tile_bytes;
         ctx->x_plan.reserve(seq_bytes + tile_bytes + (size_t)B * sizeof(int32_t));
         uint8_t* d = static_cast<uint8_t*>(ctx->x_plan.p);
-        HIP_CHECK(hipMemcpyAsync(d, seqs.data(), seq_bytes, hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipMemcpyAsync(d + seq_bytes, tiles.data(), tile_bytes, hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipMemcpyAsync(d + seq_bytes + tile_bytes, seq_of.data(), (size_t)B * sizeof(int32_t),
-                                 hipMemcpyHostToDevice, ctx->stream));
-        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // the host vectors are pageable
+        stage_upload(ctx, d, seqs.data(), seq_bytes);
+        stage_upload(ctx, d + seq_bytes, tiles.data(), tile_bytes);
+        stage_upload(ctx, d + seq_bytes + tile_bytes, seq_of.data(), (size_t)B * sizeof(int32_t));
         ctx->x_logits.reserve((size_t)logit_off * sizeof(float));
         ctx->x_sums.reserve((size_t)sum_off * sizeof(float));
         ctx->x_mask.reserve((size_t)mask_off * sizeof(uint32_t));

@@ -147,9 +147,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
 
     // The step's new K / V row of this (sequence, kv head) goes into the caches here when the step's append is fused
     // into this launch: by the wave that later reads the sequence's last block.  That wave's loads of the block must
-    // see the row: with few blocks ahead of it the wave waits for the stores before it fetches anything; otherwise the
-    // stores follow its first fetches, and at least two of its blocks -- each consumed behind a wait that covers
-    // everything issued before it -- lie between the stores and the fetch of the last block.
+    // see the row, and loads and stores of a wave may complete out of order with respect to each other, so the wave
+    // waits for its stores explicitly (vmcnt(0)) before it issues the fetch of that block: at once when the block is
+    // among its first ones, else (the stores then follow its first fetches) right in front of that fetch.
     const bool appends = a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
     const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
     auto append_rows = [&]() __attribute__((always_inline)) {
@@ -174,7 +174,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     if (tile + WAVES < te)
         issue_block<FULL, BS>(a, dsc->ids[BPT * (wv + WAVES)], dsc->ids[BPT * (wv + WAVES) + BPT - 1], (tile + WAVES) & sub_mask,
                               hkv, TILE, lane, kraw2, vraw2, traw2);
-    if (appends && !append_first) append_rows();
+    const bool append_late = appends && !append_first;
+    if (append_late) append_rows();
     // this workgroup's slice of the block table, so that no later block fetch waits on a table fetch
     int32_t* tab = reinterpret_cast<int32_t*>(smem + a.table_off);
     // (16-token blocks: two ids per tile; a last tile of one block repeats it, its second half lies beyond kv_len)
@@ -255,6 +256,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
 #pragma unroll
         for (int c = 0; c < FULL; ++c) reinterpret_cast<u4v*>(slot)[c * 64 + lane] = vr[c];
         if (lane >= 16 && lane < 32) reinterpret_cast<u4v*>(slot)[FULL * 64 + lane - 16] = tr;
+        if (append_late && tile + 2 * WAVES == tile_hi - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the appended row is in place
         if (tile + 2 * WAVES < te) {
             const int ti = BPT * (tile + 2 * WAVES - tb);
             issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], (tile + 2 * WAVES) & sub_mask, hkv, TILE, lane, kr, vr, tr);

@@ -32,6 +32,33 @@ def _check(pkg, dev, case, seed, outliers=False, want_scores=True):
     return got, ref, c
 
 
+def _outliers(torch, x, g, frac=0.01):
+    """Replaces `frac` of the elements by +-8 (the workloads' outlier recipe), in place."""
+    m = torch.rand(x.shape, generator=g, device=x.device) < frac
+    s = torch.where(torch.rand(x.shape, generator=g, device=x.device) < 0.5, 8.0, -8.0).to(x.dtype)
+    x[m] = s[m]
+    return x
+
+
+def _check_whole_batch(spec, q, kc, vc, out, scores, W, qd, kd, sw):
+    """Every sequence of a full-size workload against the checker: the blocks the tables name are gathered into a
+    compact copy of the caches (table = 0, 1, 2, ...) on the device, copied to the host, and the whole batch goes
+    through one checker call."""
+    import torch
+    O = H.O
+    Hq, Hkv, D, bs = spec["Hq"], spec["Hkv"], spec["D"], spec["bs"]
+    ids = torch.from_numpy(spec["block_indices"].astype(np.int64)).to(kc.device)
+    kcs, vcs = kc[ids].cpu().numpy(), vc[ids].cpu().numpy()
+    qs = q.view(torch.int16).cpu().numpy().view(np.uint16)
+    ref_out, _, ref_sc = O.paged_attention(
+        qs, H.DT[qd], kcs, vcs, H.DT[kd], spec["past_lens"], spec["subsequence_begins"],
+        np.arange(len(spec["block_indices"]), dtype=np.int32), spec["block_indices_begins"], Hq, Hkv, D, bs,
+        spec["scale"], sw, W, want_scores=True, num_threads=16)
+    H.assert_close(out.float().cpu().numpy(), ref_out, qd)
+    H.assert_close(scores.cpu().numpy(), ref_sc, "f16", "scores")
+
+
+
 APPEND_CASES = [("f16", "u8", 128), ("f16", "u8", 64), ("bf16", "u8", 128), ("f16", "f16", 64), ("bf16", "bf16", 128),
                 ("f16", "bf16", 128), ("bf16", "f16", 64)]
 
@@ -393,6 +420,62 @@ def test_profiling_and_split_count(pkg, dev):
         op.set_profiling(False)
 
 
+def _plant_dominant_new_rows(c, logit=16.0, v_plant=3.0):
+    """Rewrites the step's new K / V rows (single-token sequences) so that, for the first head of every kv head's
+    group, the new token takes nearly all of the softmax mass: K = q * logit / (scale |q|^2), V = a constant.  A
+    kernel that attends over the cache before its own append has landed then misses `out` by O(1) and the last score
+    by about one per kv head."""
+    from oracle import oracle as O
+    Hq, Hkv, D = c["Hq"], c["Hkv"], c["D"]
+    G = Hq // Hkv
+    qd = H.DT[c["q_dtype"]]
+    q = O.from_bits(c["query"], qd).reshape(-1, Hq, D)
+    k = np.zeros((q.shape[0], Hkv, D), np.float32)
+    for h in range(Hkv):
+        q0 = q[:, h * G, :]
+        k[:, h, :] = q0 * (logit / (c["scale"] * np.maximum((q0 * q0).sum(axis=1, keepdims=True), 1e-6)))
+    c["key"] = O.to_bits(k.reshape(q.shape[0], Hkv * D), qd)
+    c["value"] = O.to_bits(np.full((q.shape[0], Hkv * D), v_plant, np.float32), qd)
+
+
+LATE_APPEND = [
+    # (query type, cache type, block size, sequences, contexts): single-token steps in which the wave that appends a
+    # sequence's new row has fetched other tiles first; one workgroup per (sequence, kv head) and several
+    ("f16", "u8", 32, 64, (1100, 1300)), ("bf16", "u8", 16, 64, (1100, 1300)), ("f16", "u8", 64, 64, (1100, 1300)),
+    ("f16", "u8", 32, 6, (9000, 21000)), ("bf16", "u8", 32, 3, (30000, 33000)),
+    ("f16", "f16", 32, 64, (1100, 1300)), ("bf16", "bf16", 16, 64, (1100, 1300)), ("bf16", "bf16", 32, 6, (9000, 21000)),
+]
+
+
+@pytest.mark.parametrize("qd,kd,bs,B,ctx", LATE_APPEND)
+def test_fused_append_row_is_seen_by_the_launch_that_writes_it(pkg, dev, qd, kd, bs, B, ctx):
+    """The new token dominates the softmax of one head per kv head, so a stale read of its row fails `out` and
+    `scores` outright instead of hiding in the tolerance."""
+    Hq, Hkv, D = (32, 8, 128) if B >= 32 else (8, 2, 128)
+    past = np.linspace(ctx[0], ctx[1], B).astype(np.int64) | 1  # odd: the new row is never a block's first
+    case = H.case_from_lens(f"late_append_{qd}_{kd}_bs{bs}_B{B}", Hq, Hkv, D, bs, qd, kd, past, [1] * B)
+    print(f"case {case['name']}", flush=True)
+    c = H.build_case(case, 4242)
+    _plant_dominant_new_rows(c)
+    got = H.run_case_on_gpu(pkg, c, dev)
+    ref = H.run_case_on_checker(c)
+    # the step went down the path this test is about: some sequence's last workgroup walks 17 tiles or more, so the
+    # wave that owns the last tile has four tiles in front of it
+    n = got["op"].num_splits
+    tiles = (past + 1 + 31) // 32
+    per = (tiles + n - 1) // n
+    assert ((tiles - (n - 1) * per) >= 17).any(), (n, tiles.tolist())
+    assert (n > 1) == (B < 32), n
+    assert np.array_equal(got["key_cache"], ref["key_cache"]) and np.array_equal(got["value_cache"], ref["value_cache"])
+    H.assert_close(got["out"], ref["out"], qd)
+    H.assert_close(got["scores"], ref["scores"], "f16", "scores")
+    # ... and the planted rows do dominate: the first head of every group returns the planted V row
+    G = Hq // Hkv
+    o = got["out"].reshape(B, Hq, D)[:, ::G, :]
+    assert np.abs(o - 3.0).max() < 0.05, np.abs(o - 3.0).max()
+
+
+
 def test_decode_u8_ignores_garbage_beyond_the_context(pkg, dev):
     """Rows past kv_len in the last block (and unused blocks) may hold anything, NaN headers included."""
     case = H.case_from_lens("garbage_tail", 8, 2, 128, 32, "f16", "u8", [40, 90], [1, 1])
@@ -459,7 +542,8 @@ def test_errors_are_reported_not_thrown_across_the_abi(pkg, dev):
 
 
 def test_full_size_cfg2_properties(pkg, dev):
-    """Headline workload at full size: append -> attend round trip, permutation invariance, score mass."""
+    """Headline workload at full size: append -> attend round trip, permutation invariance, score mass, and the
+    whole batch against the checker."""
     import torch
     wl = __import__("openvino_genai_amd.workloads", fromlist=["x"])
     spec = wl.make_spec(2)
@@ -473,8 +557,9 @@ def test_full_size_cfg2_properties(pkg, dev):
     # fill the past by one prefill-sized append per sequence group (the product's own append, bit-exact by the tests above)
     psb = np.concatenate([[0], np.cumsum(past)]).astype(np.int32)
     Tp = int(psb[-1])
-    kp = torch.randn(Tp, Hkv * D, generator=g, device=dev, dtype=torch.float16)
-    vp = torch.randn(Tp, Hkv * D, generator=g, device=dev, dtype=torch.float16)
+    # (the workload's contents: normal values with 1 % of the elements at +-8)
+    kp = _outliers(torch, torch.randn(Tp, Hkv * D, generator=g, device=dev, dtype=torch.float16), g)
+    vp = _outliers(torch, torch.randn(Tp, Hkv * D, generator=g, device=dev, dtype=torch.float16), g)
     op.step_begin(np.zeros(B, np.int32), psb, spec["block_indices_begins"])
     op.set_block_indices(spec["block_indices"], nb)
     op.kv_append(kp, vp, kc, vc)
@@ -510,19 +595,8 @@ def test_full_size_cfg2_properties(pkg, dev):
     op.attention(q, kc2, vc2, out2, scores2)
     op.synchronize()
     assert torch.equal(out, out2) and torch.equal(scores, scores2)
-    # spot parity of one sequence against the checker at full context
-    O = H.O
-    sub = dict(B=1, Hq=Hq, Hkv=Hkv, D=D, bs=bs)
-    tab = spec["block_indices"][spec["block_indices_begins"][seq]:spec["block_indices_begins"][seq + 1]]
-    kcs = kc[torch.from_numpy(tab.astype(np.int64)).to(dev)].cpu().numpy()
-    vcs = vc[torch.from_numpy(tab.astype(np.int64)).to(dev)].cpu().numpy()
-    qs = q[seq:seq + 1].view(torch.int16).cpu().numpy().view(np.uint16)
-    ref_out, _, ref_sc = O.paged_attention(qs, O.DT_F16, kcs, vcs, O.DT_U8, past[seq:seq + 1], np.array([0, 1], np.int32),
-                                           np.arange(len(tab), dtype=np.int32), np.array([0, len(tab)], np.int32),
-                                           Hq, Hkv, D, bs, spec["scale"], 0, None, True, 8)
-    H.assert_close(out[seq:seq + 1].float().cpu().numpy(), ref_out, "f16")
-    off = int(np.sum(past[:seq] + 1))
-    H.assert_close(scores[off:off + past[seq] + 1].cpu().numpy(), ref_sc, "f16", "scores")
+    # every sequence of the batch against the checker at full context
+    _check_whole_batch(spec, q, kc, vc, out, scores, None, "f16", "u8", 0)
 
 
 def _random_case(rng, idx):
@@ -593,9 +667,9 @@ def test_peaked_single_token_row_over_u8_cache(pkg, dev):
 
 @pytest.mark.parametrize("cfg,kw", [(3, {}), (5, {}), (5, {"sliding_window": 4096}), (1, {}), (4, {})])
 def test_full_size_properties_of_the_other_workloads(pkg, dev, cfg, kw):
-    """Full-size workloads beyond the checker's reach: append -> attend, score mass per sequence (every softmax row
+    """Full-size workloads: append -> attend, score mass per sequence (every softmax row
     sums to one, so a sequence's scores sum to Hq x W), zero scores outside the sliding window, identical bits under
-    another physical placement of the blocks, and spot parity of single sequences against the checker."""
+    another physical placement of the blocks, and the whole batch against the checker."""
     import torch
     wl = __import__("openvino_genai_amd.workloads", fromlist=["x"])
     spec = wl.make_spec(cfg, **kw)
@@ -647,14 +721,5 @@ def test_full_size_properties_of_the_other_workloads(pkg, dev, cfg, kw):
     op.attention(q, kc[perm], vc[perm], out2, scores2)
     op.synchronize()
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16)) and torch.equal(scores, scores2)
-    # spot parity: the shortest and the longest sequence, each alone, against the checker
-    O = H.O
-    for b in (int(np.argmin(past + new)), int(np.argmax(past + new))):
-        tab = torch.from_numpy(spec["block_indices"][bib[b]:bib[b + 1]].astype(np.int64)).to(dev)
-        qs = q[sb[b]:sb[b + 1]].view(torch.int16).cpu().numpy().view(np.uint16)
-        ref_out, _, ref_sc = O.paged_attention(
-            qs, H.DT[qd], kc[tab].cpu().numpy(), vc[tab].cpu().numpy(), H.DT[kd], past[b:b + 1],
-            np.array([0, new[b]], np.int32), np.arange(len(tab), dtype=np.int32), np.array([0, len(tab)], np.int32),
-            Hq, Hkv, D, bs, spec["scale"], sw, W[b:b + 1], want_scores=True, num_threads=16)
-        H.assert_close(out[sb[b]:sb[b + 1]].float().cpu().numpy(), ref_out, qd)
-        H.assert_close(sc[off[b]:off[b + 1]], ref_sc, "f16", "scores")
+    # every sequence of the batch against the checker (config 3's chunks are a minute of checker time)
+    _check_whole_batch(spec, q, kc, vc, out, scores, W, qd, kd, sw)

@@ -26,10 +26,9 @@ NUM_LAYERS_FOR_TOKS = 32  # Llama-3-8B depth: tok/s = batch / (32 * t_layer), at
 
 # HBM bytes per launch of the dominant kernel: not measured by this script but read off rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of it, scaled by the readings of a plain 1 GiB copy; the summary file holds commands and readings.
+# (a workload without a reading of the kernel as it stands is not listed: `traffic` is then null)
 MEASURED_TRAFFIC = {
     "llama3_8b_decode_u8_b64_ctx4096": (585.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
-    "llama3_8b_eviction_u8_b256_ctx8192": (4655.0e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
-    "long_context_decode_u8_b8_ctx32768": (594.3e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
     "qwen25_7b_mixed_bf16": (835.0e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
 }
 
@@ -437,17 +436,23 @@ def main():
     def step():
         op.forward(q, k, v, kc, vc, out, scores)
 
+    def timed_steps():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize(dev)
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # The same W + K steps first as a fresh process finds the GPU (clocks not yet settled), reported beside the
+    # settled figure so that the record shows how much of it is the kernel and how much the clocks.
+    unsettled_ms = timed_steps() if args.settle_steps > 0 else None
     for _ in range(args.settle_steps):  # clocks settle; not part of the warmup, not timed
         step()
     torch.cuda.synchronize(dev)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize(dev)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize(dev)
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed_steps()
 
     # the dominant kernel alone: the library brackets it with HIP events on its launch stream
     op.set_profiling(True)
@@ -509,6 +514,15 @@ def main():
     }
     res["roofline"]["ms_p10_p50_p90"] = [round(p10, 5), round(p50, 5), round(p90, 5)]
     res["roofline"]["ms_mean"] = round(attn_mean_ms, 5)
+    # `frac` prices the median launch; the same fraction from the mean of the launches beside it
+    res["roofline"]["frac_p50"] = res["roofline"]["frac"]
+    res["roofline"]["frac_mean"] = round(res["roofline"]["frac"] * attn_ms / attn_mean_ms, 4)
+    if unsettled_ms is not None:
+        res["unsettled"] = {"ms_per_step": round(unsettled_ms, 5),
+                            "value": round(bytes_["total"] / (unsettled_ms * 1e-3) / 1e9, 1),
+                            "pct_hbm_peak": round(100.0 * bytes_["total"] / (unsettled_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                            "note": "the same %d warm-up + %d timed steps run first, before the %d settle steps: what a "
+                                    "fresh process measures while the clocks still ramp" % (args.warmup, args.steps, args.settle_steps)}
     res["roofline"]["launches"] = len(kernel_ms)
     if cold_ms:
         cold = float(np.median(cold_ms))

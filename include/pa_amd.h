@@ -322,7 +322,14 @@ int32_t pa_evictor_reset_slot(pa_evictor* ev, int32_t slot);
 
 /* register_new_token_scores for a batch of sequences: `scores_per_layer` is a host array of
  * num_decoder_layers device pointers (`scores.<L>`); sequence i's vector is
- * [offsets[i], offsets[i+1]) in each of them; num_snapkv_scores may be NULL (all 0). */
+ * [offsets[i], offsets[i+1]) in each of them; num_snapkv_scores may be NULL (all 0).
+ * The call returns once its kernel is QUEUED on the evictor's stream: the host arrays are free again, the
+ * `scores.<L>` device tensors are read later, in stream order.  Work that follows on the same stream (the next
+ * step's pa_forward rewriting the tensors, pa_evictor_evict, ...) is ordered behind that read by the stream
+ * itself; rewriting the tensors from ANOTHER stream needs an event or a synchronisation in between, and so does
+ * producing them on another stream than the evictor's (give the evictor the pa_ctx's stream).  Of the pair
+ * register / evict, register returns with its work in flight, pa_evictor_evict returns synchronised (its lists are
+ * host arrays). */
 int32_t pa_evictor_register_scores(pa_evictor* ev, int32_t num_sequences, const int32_t* slots,
                                    const float* const* scores_per_layer, const int64_t* offsets,
                                    const uint64_t* num_snapkv_scores);

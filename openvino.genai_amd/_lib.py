@@ -6,7 +6,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SO_PATH = os.path.join(_HERE, "csrc", "libpa_amd.so")
+# PA_AMD_LIBRARY names another build of the library (one with instrumentation, say); it must export the same C-ABI
+SO_PATH = os.environ.get("PA_AMD_LIBRARY") or os.path.join(_HERE, "csrc", "libpa_amd.so")
 
 PA_OK = 0
 PA_F16, PA_BF16, PA_U8 = 0, 1, 2

@@ -89,6 +89,17 @@ __device__ __forceinline__ float xor_sum_g(float v) {
     return a + b;
 }
 
+// acc + the two 16-bit floats of `w` (one instruction: a dot product with (1, 1))
+template <int DT>
+__device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+    if (DT == DT_F16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w), __builtin_bit_cast(h2, 0x3c003c00u), acc, false);
+    }
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, w), __builtin_bit_cast(b2, 0x3f803f80u), acc, false);
+}
+
 // f32 -> cache-type bits, two values at a time
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
@@ -310,6 +321,12 @@ void pa_prefill16_kernel(PrefillArgs a) {
     }
 
     float m_run[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.0f, 0.0f};
+    // 16-bit caches keep the running maximum negated (NO_MAX while the row has seen nothing), ready for the exponent's
+    // multiply-add, and the level (log2, relative to the running maximum) a block's largest probability must stay
+    // under for the block to do without the second, low-half product: log2(LO_SHARE x the row's denominator when
+    // last looked at).
+    constexpr float NO_MAX = 1e30f;
+    float neg_m[2] = {NO_MAX, NO_MAX}, lo_at[2] = {-INFINITY, -INFINITY};
     float zsum[2] = {0.0f, 0.0f};  // u8: this lane's share of sum_t w_t zp_v
     f4 acc[2][RT];
 #pragma unroll
@@ -480,7 +497,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
             }
         }
     };
-    // masks + online softmax of block `tile` (number j): probabilities as MFMA operands, rescale factors.
+    // u8 caches: masks + online softmax of block `tile` (number j): weights as MFMA operands, rescale factors.
     // The running maximum is only raised when a block exceeds it by more than 2^4: probabilities then stay
     // below 16 and the accumulators are rescaled a few times per row instead of once per block.
     auto softmax = [&](auto masked_c, const f4 (&sc)[2][2], int tile, int j, u4v (&pb)[2], u4v (&pl)[2],
@@ -508,9 +525,6 @@ void pa_prefill16_kernel(PrefillArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                         x[4 * u + i] = fmaf(sc[gi][u][i] * (scl * CODE_UNIT), h_sck[u][i], -h_zpk[u][i] * qsum[gi]);
-            } else {  // raw dot products: the scale is folded into the exponent's multiply-add below
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) x[jj] = sc[gi][jj >> 2][jj & 3];
             }
             if (MASKED) {
                 const int lim = row_pos[gi];
@@ -523,7 +537,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
             }
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) mx = fmaxf(mx, x[jj]);
-            mx = xor_max_g(mx) * (U8 ? 1.0f : scl);
+            mx = xor_max_g(mx);
             const float m_new = mx > m_run[gi] + 4.0f ? mx : m_run[gi];
             const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
             corr[gi] = __builtin_amdgcn_exp2f(m_run[gi] - m_safe);
@@ -531,7 +545,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
             float psum = 0.0f;
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) {
-                p[jj] = __builtin_amdgcn_exp2f(U8 ? x[jj] - m_safe : fmaf(x[jj], scl, -m_safe));
+                p[jj] = __builtin_amdgcn_exp2f(x[jj] - m_safe);
                 psum += p[jj];
             }
             if (U8) {
@@ -558,20 +572,79 @@ void pa_prefill16_kernel(PrefillArgs a) {
                 }
                 zsum[gi] = zsum[gi] * corr[gi] + zs;
             }
+            l_part[gi] = l_part[gi] * corr[gi] + psum;
+            m_run[gi] = m_new;
+        }
+    };
+
+    // ---- 16-bit caches: the softmax of a block, and the product with the probabilities --------------------------
+    // Probabilities enter the matrix pipe rounded to the cache type, as a high half and -- what that rounding dropped --
+    // a low half: 16 significant bits for bf16, 22 for f16.  With the high half alone (8 bits for bf16) the rounding
+    // of a single dominant token's probability is outside the tolerance whenever large V values of opposite sign
+    // cancel.  The denominator is the sum of the rounded halves (one dot-product instruction per pair), so a row's
+    // weights stay a convex combination whatever the rounding did.
+    // f16 caches: 11 bits are enough for every token that is a small share of its row, so the low halves follow only
+    // for blocks in which some row has a token whose probability exceeds 2^LO_SHARE_LOG2 of that row's denominator so
+    // far (the running one, a lower bound of the final one).  The rounding errors of the tokens below that share add
+    // up like noise of at most 2^-12 sqrt(share) x the spread of V per row; a row that leans on a few tokens -- where
+    // one rounding error is the whole error -- takes both halves.  bf16 caches always take both: at 8 bits the share
+    // would have to be so small that nearly every block of a context of a few thousand tokens exceeds it.
+    // Returns (wave-uniform) whether this block needs the low halves.
+    constexpr bool LO_ALWAYS = DT == DT_BF16;
+    constexpr float LO_SHARE_LOG2 = -2.0f;
+    auto softmax16 = [&](auto masked_c, const f4 (&sc)[2][2], int tile, int j, u4v (&pb)[2], float (&p)[2][8],
+                         const bool (&kept)[2]) __attribute__((always_inline)) -> bool {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        const int pos0 = tile * TOK + 4 * g;
+        float x[2][8], mxs[2], rel[2];  // rel: the block's maximum relative to the running one (huge while there is none)
+        bool raise = false;
 #pragma unroll
-            for (int jj = 0; jj < (U8 ? 0 : 4); ++jj) {
-                // second operand: what the rounding to the operand type dropped
-                uint32_t hi = pack2<DT>(p[2 * jj], p[2 * jj + 1]);
+        for (int gi = 0; gi < NG; ++gi) {
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) x[gi][jj] = sc[gi][jj >> 2][jj & 3];  // raw dot products: the scale is folded into the exponent's multiply-add
+            if (MASKED) {
+                const int lim = row_pos[gi];
+                const int low = sw > 0 ? max(0, lim + 1 - sw) : 0;
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj) {
+                    const int pos = pos0 + 16 * (jj >> 2) + (jj & 3);
+                    x[gi][jj] = (pos <= lim && pos >= low && kept[gi]) ? x[gi][jj] : -INFINITY;
+                }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) mx = fmaxf(mx, x[gi][jj]);
+            mxs[gi] = xor_max_g(mx) * scl;
+            rel[gi] = mxs[gi] + neg_m[gi];  // (-inf for a row that sees nothing of this block)
+            raise |= rel[gi] > 4.0f;
+        }
+        // The running maximum is only raised when a block exceeds it by more than 2^4: probabilities then stay below
+        // 16 and the accumulators are rescaled a few times per row instead of once per block.
+        if (__any(raise)) {
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) {
+                const float m_new = rel[gi] > 4.0f ? mxs[gi] : -neg_m[gi];
+                const float d = -neg_m[gi] - m_new;  // 0 for a row that stays; -NO_MAX for one that held nothing (zeros)
+                const float corr = __builtin_amdgcn_exp2f(d);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) acc[gi][r] *= corr;
+                l_part[gi] *= corr;
+                lo_at[gi] += d;
+                neg_m[gi] = -m_new;
+                rel[gi] = mxs[gi] + neg_m[gi];
+            }
+        }
+        bool need = false;
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) p[gi][jj] = __builtin_amdgcn_exp2f(fmaf(x[gi][jj], scl, neg_m[gi]));
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                uint32_t hi = pack2<DT>(p[gi][2 * jj], p[gi][2 * jj + 1]);
                 if (DT == DT_BF16) asm("" : "+v"(hi));  // (its halves are taken from this word, not converted once more)
                 pb[gi][jj] = hi;
-                if (DT == DT_BF16) {
-                    pl[gi][jj] = pack2<DT>(p[2 * jj] - __builtin_bit_cast(float, hi << 16),
-                                           p[2 * jj + 1] - __builtin_bit_cast(float, hi & 0xffff0000u));
-                } else {
-                    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-                    const h2 h = __builtin_bit_cast(h2, hi);
-                    pl[gi][jj] = pack2<DT>(p[2 * jj] - (float)h[0], p[2 * jj + 1] - (float)h[1]);
-                }
+                l_part[gi] = add_pair<DT>(hi, l_part[gi]);
                 if constexpr (STASH) {
                     if (emit && gi == 0) {
                         // (head and token group of the lane from an opaque copy of the thread id: kept in registers of
@@ -582,15 +655,54 @@ void pa_prefill16_kernel(PrefillArgs a) {
                         const int ne = te_ & 15, ge = (te_ >> 4) & 3;
                         if (ne < G) {
                             uint8_t* at = pkeep + ((j * G + ne) * TOK + 4 * ge + 16 * (jj >> 1) + 2 * (jj & 1)) * 2;
-                            *reinterpret_cast<uint32_t*>(at) = pack2<DT_F16>(p[2 * jj], p[2 * jj + 1]);
-                            if (jj == 0 && ge == 0)
-                                *reinterpret_cast<float*>(pkeep + single_item_max_tiles(G) * G * TOK * 2 + (j * G + ne) * 4) = m_safe;
+                            *reinterpret_cast<uint32_t*>(at) = pack2<DT_F16>(p[gi][2 * jj], p[gi][2 * jj + 1]);
+                            if (jj == 0 && ge == 0)  // (a single-token row sees its item's first block, so it has a maximum)
+                                *reinterpret_cast<float*>(pkeep + single_item_max_tiles(G) * G * TOK * 2 + (j * G + ne) * 4) = -neg_m[gi];
                         }
                     }
                 }
             }
-            l_part[gi] = l_part[gi] * corr[gi] + psum;
-            m_run[gi] = m_new;
+            need |= rel[gi] > lo_at[gi];
+        }
+        if constexpr (LO_ALWAYS) return true;
+        if (!__any(need)) return false;
+        // some row's largest probability is above the share of the denominator it was last compared with: look at the
+        // denominators as they are now (this block included)
+        need = false;
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            lo_at[gi] = __log2f(xor_sum_g(l_part[gi])) + LO_SHARE_LOG2;
+            need |= rel[gi] > lo_at[gi];
+        }
+        return __any(need);
+    };
+    // what the rounding of the probabilities dropped, as operands of their own (and into the denominator)
+    auto make_lo = [&](const u4v (&pb)[2], const float (&p)[2][8], u4v (&pl)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const uint32_t hi = pb[gi][jj];  // (a bit cast straight from a vector element reads element 0)
+                uint32_t lo;
+                if (DT == DT_BF16) {
+                    lo = pack2<DT>(p[gi][2 * jj] - __builtin_bit_cast(float, hi << 16),
+                                   p[gi][2 * jj + 1] - __builtin_bit_cast(float, hi & 0xffff0000u));
+                } else {
+                    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                    const h2 h = __builtin_bit_cast(h2, hi);
+                    lo = pack2<DT>(p[gi][2 * jj] - (float)h[0], p[gi][2 * jj + 1] - (float)h[1]);
+                }
+                pl[gi][jj] = lo;
+                l_part[gi] = add_pair<DT>(lo, l_part[gi]);
+            }
+    };
+    // O^T += V^T . P^T with one set of probability operands: sixteen (eight) independent accumulator tiles in a row
+    auto pv_only = [&](const uint8_t* vb, const u4v (&pp)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const s8v vop = load_v(vb, r);
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) acc[gi][r] = mma<DT>(vop, __builtin_bit_cast(s8v, pp[gi]), acc[gi][r]);
         }
     };
 
@@ -599,17 +711,31 @@ void pa_prefill16_kernel(PrefillArgs a) {
                           __attribute__((always_inline)) {
         f4 sc[2][2];
         u4v pb[2], pl[2];
-        float corr[2];
-        qk_pv_at(true, kb, sc, false, vb, pb, pl);
-        softmax(masked_c, sc, tile_at(j), j, pb, pl, corr, kept);
+        if constexpr (U8) {
+            float corr[2];
+            qk_pv_at(true, kb, sc, false, vb, pb, pl);
+            softmax(masked_c, sc, tile_at(j), j, pb, pl, corr, kept);
 #pragma unroll
-        for (int gi = 0; gi < NG; ++gi) {
-            if (__any(corr[gi] != 1.0f)) {
+            for (int gi = 0; gi < NG; ++gi) {
+                if (__any(corr[gi] != 1.0f)) {
 #pragma unroll
-                for (int r = 0; r < RT; ++r) acc[gi][r] *= corr[gi];
+                    for (int r = 0; r < RT; ++r) acc[gi][r] *= corr[gi];
+                }
+            }
+            qk_pv_at(false, kb, sc, true, vb, pb, pl);
+        } else {
+            float p[2][8];
+            qk_pv_at(true, kb, sc, false, vb, pb, pl);
+            const bool lo = softmax16(masked_c, sc, tile_at(j), j, pb, p, kept);
+            if constexpr (LO_ALWAYS) {  // both halves in one stream, each V operand read once
+                make_lo(pb, p, pl);
+                qk_pv_at(false, kb, sc, true, vb, pb, pl);
+            } else {
+                if (lo) make_lo(pb, p, pl);
+                pv_only(vb, pb);
+                if (lo) pv_only(vb, pl);
             }
         }
-        qk_pv_at(false, kb, sc, true, vb, pb, pl);
     };
     auto whole_at = [&](int j, const uint8_t* kb, const uint8_t* vb) __attribute__((always_inline)) {
         const int tile = tile_at(j);
@@ -633,30 +759,44 @@ void pa_prefill16_kernel(PrefillArgs a) {
     if constexpr (DMA) {
         // Block number j lives in K slot and V slot j % 4.  A wave moves rows 8 wv .. 8 wv + 7 of a block: lane l of
         // its two instructions per tensor takes row 8 wv + 4 i + l / 16, LDS piece position l % 16, i.e. the row's
-        // piece (l % 16) ^ (row & 15).  Every step issues the same four copies per wave (indices clamped), so that
-        // "at most eight outstanding" always means: everything but the two youngest blocks has landed.
-        const int my_row = 8 * wv + (lane >> 4);          // + 4 for the second instruction
-        const int my_piece = ((lane & 15) ^ (my_row & 15)) << 4;
-        const int my_piece2 = ((lane & 15) ^ ((my_row + 4) & 15)) << 4;
-        const int my_vpiece = ((lane & 15) ^ ((my_row & 7) << 1)) << 4;
-        const int my_vpiece2 = ((lane & 15) ^ (((my_row + 4) & 7) << 1)) << 4;
-        // (the block id of a copy is read one step before the copy goes out: a scalar load that is waited for right behind
-        // its issue stalls the wave at the start of every step)
-        const bool upper_half = __builtin_amdgcn_readfirstlane(wv) >= (NT / 64) / 2;  // this wave moves rows 16 - 31
-        long base_next = 0;
-        auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
-            const long blk = base_next;
-            base_next = tile_base(tile_at(j + 1), upper_half);
-            const uint8_t* kg = a.key_cache + blk + my_row * ROWB;
-            const uint8_t* vg = a.value_cache + blk + my_row * ROWB;
-            uint8_t* kd = kslot_base + wv * 2048;
-            uint8_t* vd = vslot_base + wv * 2048;
-            dma16(kg + my_piece, kd);
-            dma16(kg + 4 * ROWB + my_piece2, kd + 1024);
-            dma16(vg + my_vpiece, vd);
-            dma16(vg + 4 * ROWB + my_vpiece2, vd + 1024);
+        // piece (l % 16) ^ (row & 15) of K, (l % 16) ^ 2 (row & 7) of V.  Every step issues the same four copies per
+        // wave (indices clamped), so that "at most eight outstanding" always means: everything but the two youngest
+        // blocks has landed.
+        const int wvs = __builtin_amdgcn_readfirstlane(wv);
+        const int my_row = 8 * wvs + (lane >> 4);         // + 4 for the second instruction
+        // per-lane byte offsets within a block (32 bits, added to a wave-uniform block address)
+        const uint32_t off_k0 = my_row * ROWB + (((lane & 15) ^ (my_row & 15)) << 4);
+        const uint32_t off_k1 = (my_row + 4) * ROWB + (((lane & 15) ^ ((my_row + 4) & 15)) << 4);
+        const uint32_t off_v0 = my_row * ROWB + (((lane & 15) ^ ((my_row & 7) << 1)) << 4);
+        const uint32_t off_v1 = (my_row + 4) * ROWB + (((lane & 15) ^ (((my_row + 4) & 7) << 1)) << 4);
+        const bool upper_half = wvs >= (NT / 64) / 2;  // this wave moves rows 16 - 31
+        // The table entry of a copy's block is read one step before the copy goes out, and nothing is computed from it
+        // until then: a scalar load that is waited for right behind its issue stalls the wave at every step.
+        auto table_index = [&](int tile) __attribute__((always_inline)) {
+            return bs16 ? min(2 * tile + (upper_half ? 1 : 0), last_block16) : tile >> sub_shift;
         };
-        base_next = tile_base(tile_at(0), upper_half);
+        int id_next = table[table_index(tile_at(0))];
+        auto copy_in = [&](int j, uint8_t* kslot_base, uint8_t* vslot_base) __attribute__((always_inline)) {
+            const int tile = tile_at(j);
+            // (what tile_base gives for this wave's half of the tile, from the entry read a step ago)
+            const long blk = bs16 ? ((long)id_next * Hkv + hkv) * (16 * CROWB) - (upper_half ? 16 * CROWB : 0)
+                                  : ((long)id_next * Hkv + hkv) * ((long)a.sh.bs * CROWB) + (long)(tile & sub_mask) * (TOK * CROWB);
+            id_next = table[table_index(tile_at(j + 1))];
+            const uint8_t* kg = a.key_cache + blk;
+            const uint8_t* vg = a.value_cache + blk;
+            uint8_t* kd = kslot_base + wvs * 2048;
+            uint8_t* vd = vslot_base + wvs * 2048;
+            dma16(kg + off_k0, kd);
+            dma16(kg + off_k1, kd + 1024);
+            dma16(vg + off_v0, vd);
+            dma16(vg + off_v1, vd + 1024);
+        };
+        // The wait in front of a step's barrier names how many of the wave's vector-memory operations may still be
+        // outstanding: the copies of the two youngest blocks.  It is only right while a step issues exactly this many
+        // copies per wave and nothing else that counts (the table reads above are scalar loads; the build fails on
+        // spills, whose scratch traffic would count).
+        constexpr int COPIES_PER_STEP = 4;
+        static_assert(COPIES_PER_STEP == 2 * (TOK * ROWB / 1024) / (NT / 64), "copy_in issues one 1024-byte copy per 8 rows of K and of V for each wave");
         copy_in(0, dk0, dv0);
         copy_in(1, dk1, dv1);
         copy_in(2, dk2, dv2);
@@ -669,7 +809,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
 #define PA_DMA_STEP(kc, vc, kn, vn)                                                                      \
         {                                                                                                \
             if (j >= cnt) break;                                                                         \
-            wait_vmem<8>();  /* this wave's part of block j has landed (blocks j + 1, j + 2 may be on their way) */ \
+            wait_vmem<2 * COPIES_PER_STEP>();  /* this wave's part of block j has landed (blocks j + 1, j + 2 may be on their way) */ \
             lds_barrier();   /* so has everyone else's, and block j - 1 is done with */                  \
             copy_in(j + 3, kn, vn);                                                                      \
             const int tile = tile_at(j);                                                                 \
@@ -755,6 +895,10 @@ void pa_prefill16_kernel(PrefillArgs a) {
     }
 
     // ---- write the rows ------------------------------------------------------------------------------
+    if constexpr (!U8) {
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) m_run[gi] = neg_m[gi] == NO_MAX ? -INFINITY : -neg_m[gi];
+    }
     const bool final_out = item.nsplit == 1;
     // the lane's group number again, from an opaque copy of the thread id: nothing inside the loop reads it, and kept
     // alive across the loop it costs the variants that sit at their register limit a spill

@@ -137,6 +137,41 @@ def test_batched_decode_steps_match_checker_exactly(pkg, mode, snapkv):
     assert any(len(b) for b in got[0]) or True
 
 
+@pytest.mark.parametrize("mode", ["NORM_SUM", "ADAPTIVE_RKV"])
+def test_scores_may_be_rewritten_in_stream_order_right_after_registering(pkg, mode):
+    """pa_evictor_register_scores returns with its kernel queued: the score tensors are read in stream order, so work
+    queued behind the call on the same stream -- here a fill that overwrites them at once, many times over a large
+    registration -- must not reach what the registration reads."""
+    import torch
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(77)
+    B, L, bs = 6, 4, 32
+    m = pkg.AggregationMode[mode]
+    rkv = {"adaptive_rkv_window_size": 4, "attention_mass": 0.9} if mode == "ADAPTIVE_RKV" else {}
+    cfg = (pkg.CacheEvictionConfig(32, 128, 1024, m, False, 0, None, pkg.AdaptiveRKVConfig(0.9, 4)) if rkv else
+           pkg.CacheEvictionConfig(32, 128, 1024, m, False, 0))
+    ev = pkg.Evictor(cfg, bs, L, 7, max_sequences=B, max_tracked_tokens=40000, device=0,
+                     stream=torch.cuda.current_stream(dev))
+    refs = [O.CacheEvictionAlgorithm(32, 128, 1024, int(m), 0, bs, L, 7, **rkv) for _ in range(B)]
+    slots = np.arange(B, dtype=np.int32)
+    lens = rng.integers(30000, 36000, B)
+    offsets = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    bufs = [torch.empty(int(offsets[-1]), dtype=torch.float32, device=dev) for _ in range(L)]
+    for step in range(4):
+        host = [rng.random(int(offsets[-1])).astype(np.float32) for _ in range(L)]
+        for t, h in zip(bufs, host):
+            t.copy_(torch.from_numpy(h).to(dev))
+        ev.register_new_token_scores(slots, [t.data_ptr() for t in bufs], offsets, None)
+        for t in bufs:  # queued behind the registration on the same stream, no synchronisation in between
+            t.fill_(float("nan"))
+        for i in range(B):
+            refs[i].register_new_token_scores([h[offsets[i]:offsets[i + 1]] for h in host], (), 0)
+    for i in range(B):
+        for l in range(L):
+            gs, gc = ev.get_state(i, l)
+            assert np.array_equal(gs, refs[i].get_scores()[l]), (i, l)
+
+
 def test_evictor_rejects_bad_calls(pkg):
     import torch
     ev = pkg.Evictor(pkg.CacheEvictionConfig(32, 32, 192, pkg.AggregationMode.NORM_SUM, False, 4), 4, 2, 1,

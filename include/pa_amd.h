@@ -36,8 +36,8 @@ enum {
     PA_UNKNOWN_EXCEPTION = -17
 };
 
-/* element types of the tensors the op sees */
-enum { PA_F16 = 0, PA_BF16 = 1, PA_U8 = 2 };
+/* element types of the tensors the op sees.  PA_U4 (cache tensors only): 4-bit codes, two per byte */
+enum { PA_F16 = 0, PA_BF16 = 1, PA_U8 = 2, PA_U4 = 3 };
 
 /* AggregationMode, include/openvino/genai/cache_eviction.hpp:19-26 */
 enum { PA_AGG_SUM = 0, PA_AGG_NORM_SUM = 1, PA_AGG_ADAPTIVE_RKV = 2 };
@@ -65,14 +65,23 @@ typedef struct pa_config {
     int32_t device;          /* HIP device ordinal */
     int32_t num_heads;       /* query heads */
     int32_t num_kv_heads;    /* KV heads; num_heads must be a multiple */
-    int32_t head_size;       /* 64 or 128 */
+    int32_t head_size;       /* elements of a query / key row: a multiple of 8 up to 512 (64 and 128 have tuned kernels) */
     int32_t block_size;      /* tokens per KV block: the reference fixes 32 on CPU, 16 on GPU
                                 (kv_cache_manager.hpp:97-110); here a knob */
     int32_t query_dtype;     /* PA_F16 | PA_BF16: query, key, value and the output */
-    int32_t kv_cache_dtype;  /* PA_U8 | PA_F16 | PA_BF16: what ov::hint::kv_cache_precision resolves to
-                                (src/cpp/src/utils.cpp:840-863) */
+    int32_t kv_cache_dtype;  /* PA_U8 | PA_U4 | PA_F16 | PA_BF16: what ov::hint::kv_cache_precision resolves to
+                                (src/cpp/src/utils.cpp:840-863); the key cache's type, and the value cache's unless
+                                value_cache_dtype_p1 says otherwise */
     int32_t num_layers;      /* decoder layers (block tables may differ per layer with eviction) */
     void* stream;            /* hipStream_t to launch on; NULL = the device's default stream */
+    /* The value side where it differs from the key side: a model's value_cache.<L> may have another head size and
+     * another precision than its key_cache.<L> (the reference keeps shape and precision per tensor,
+     * src/cpp/src/continuous_batching/cache/kv_cache_manager.hpp:74-92, and reads the V head size on its own,
+     * :274-276).  Zero in either field = as the key side, so a zero-initialised tail keeps the old meaning.  Shapes and
+     * precisions that differ from layer to layer take one pa_ctx per distinct combination (contexts are cheap; they
+     * share nothing but the device). */
+    int32_t v_head_size;            /* elements of a value / output row; 0 = head_size */
+    int32_t value_cache_dtype_p1;   /* 0 = kv_cache_dtype, else 1 + (PA_U8 | PA_U4 | PA_F16 | PA_BF16) */
 } pa_config;
 
 /* Replaces Core::compile_model + create_infer_request for this op (pipeline_impl.cpp:182,193). */
@@ -104,12 +113,14 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* meta);
 int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* block_indices, int32_t count,
                              int64_t num_blocks);
 
-/* Tensors of one layer's call, all in device memory:
- *   query [T, Hq*D], key/value [T, Hkv*D] in query_dtype;
- *   key_cache/value_cache [num_blocks, Hkv, block_size, row] in kv_cache_dtype, where a row is D
- *   elements for f16/bf16 and `f32 scale | f32 zero-point | D codes` (D+8 bytes) for u8
- *   (`key_cache.<L>` / `value_cache.<L>`, kv_cache_manager.hpp:30-33);
- *   out [T, Hq*D] in query_dtype; scores f32 [sum_b(past_b + new_b)] or NULL (`scores.<L>`,
+/* Tensors of one layer's call, all in device memory (D = head_size, Dv = the value head size):
+ *   query [T, Hq*D], key [T, Hkv*D], value [T, Hkv*Dv] in query_dtype;
+ *   key_cache [num_blocks, Hkv, block_size, row of D elements], value_cache [.., row of Dv elements], each in its
+ *   cache type: a row of n elements is n 16-bit values for f16 / bf16, `f32 scale | f32 zero-point | n codes`
+ *   (n + 8 bytes) for u8 and `f32 scale | f32 zero-point | n / 2 bytes` (element 2 i in the high nibble of byte i)
+ *   for u4 (`key_cache.<L>` / `value_cache.<L>`, kv_cache_manager.hpp:30-33; the u4 row format is this library's
+ *   reading of the plugin's, which the reference tree does not hold);
+ *   out [T, Hq*Dv] in query_dtype; scores f32 [sum_b(past_b + new_b)] or NULL (`scores.<L>`,
  *   model_runner.hpp:23-27, 1518-1568). */
 typedef struct pa_layer_io {
     const void* query;
@@ -122,10 +133,14 @@ typedef struct pa_layer_io {
     float* scores;
 } pa_layer_io;
 
-/* One layer's PagedAttention: KV append (+ u8 quantisation), attention, optional scores.  The op's `alibi_slopes`
+/* One layer's PagedAttention: KV append (+ u8 / u4 quantisation), attention, optional scores.  The op's `alibi_slopes`
  * input has no counterpart: no ALiBi term is applied, and a binding must refuse a non-empty slopes tensor.  Tuned
- * kernels serve block_size 16, 32, 64, 128 and 256, head size 64 / 128; other shapes run on a generic kernel.  In a step whose sequences all schedule one token (u8 cache, or an f16 / bf16 cache of the query's type) the append
- * is done by the attention kernel itself (the cache rows are the ones pa_kv_append writes). */
+ * kernels serve block_size 16, 32, 64, 128 and 256 with head size 64 or 128, K and V alike, over a u8 cache or an f16 /
+ * bf16 cache of the query's type; every other combination pa_create accepts (other head sizes, a value head size or
+ * value precision of its own, u4 rows, a 16-bit cache of the other 16-bit type, other block sizes) runs on shape-generic
+ * kernels, correct but far from the tuned ones' speed.  In a step whose sequences all schedule one token, over a cache
+ * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
+ * writes). */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The two halves of pa_forward on their own (same arguments; pa_kv_append ignores query/out/scores,
  * pa_attention ignores key/value). */
@@ -133,8 +148,9 @@ int32_t pa_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* pa_attention for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as pa_attention, for steps
- * in which every sequence schedules one token, over a u8 cache or a 16-bit cache of the query's type (block size 32,
- * head size 64 or 128, at most 16 query heads per kv head); other steps return PA_NOT_IMPLEMENTED.  The split partials,
+ * in which every sequence schedules one token, over a u8 cache or a 16-bit cache of the query's type (block size 16 to
+ * 256, a power of two; head size 64 or 128, K and V alike; at most 16 query heads per kv head); other steps return
+ * PA_NOT_IMPLEMENTED.  The split partials,
  * final maxima / denominators and the score staging live in a fixed device array of PA_STATIC_SCRATCH_BYTES bytes
  * (32 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls
  * no hipMalloc / hipFree; a step that needs more returns PA_OUT_OF_BOUNDS and a message with the byte count.  (The
@@ -232,8 +248,9 @@ float pa_xattention_threshold(float configured_threshold, uint64_t num_last_dens
  *     its groups; tokens outside the chunk count as zero vectors;
  *   - per (query head, I): key blocks 0 and I are kept, then the others in descending importance until the kept sum
  *     reaches threshold * the row's sum; a query row then sees a key position only if its block pair was kept.
- * Needs block_size 32 caches, head_size 64 / 128, a u8 cache or one of the query's type; xattention_block_size a
- * power of two >= 32, xattention_stride a power of two <= 32 (PA_NOT_IMPLEMENTED otherwise). */
+ * Needs a cache block_size of 32, 64, 128 or 256, head_size 64 / 128 (K and V alike), a u8 cache or one of the query's
+ * type; xattention_block_size a power of two >= 32, xattention_stride a power of two <= 32 (PA_NOT_IMPLEMENTED
+ * otherwise). */
 int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t xattention_block_size,
                           int32_t xattention_stride);
 /* Diagnostics of the last pa_attention / pa_forward call of the step (no counterpart in the reference, whose op keeps
@@ -257,7 +274,25 @@ uint64_t pa_snapkv_num_scores(uint64_t snapkv_window_size, uint64_t prompt_len, 
  * ---------------------------------------------------------------------------------------------- */
 typedef struct pa_kv_cache pa_kv_cache;
 
+/* One cache tensor as the reference reads it off the model's `key_cache.<L>` / `value_cache.<L>` input: shape
+ * [num_blocks, num_kv_heads, block_size, head_size] and element type (kv_cache_manager.hpp:74-92).  Any PA_* cache
+ * type; sub-byte types halve the bytes (kv_cache_manager.hpp:152-157). */
+typedef struct pa_kv_tensor_desc {
+    int32_t num_kv_heads;
+    int32_t block_size;
+    int32_t head_size;
+    int32_t dtype;
+} pa_kv_tensor_desc;
+typedef struct pa_kv_layer_desc {
+    pa_kv_tensor_desc key, value;
+} pa_kv_layer_desc;
+
+/* every layer alike, from the op's configuration (value side included) */
 int32_t pa_kv_cache_create(const pa_config* cfg, pa_kv_cache** out);
+/* shape and precision per layer and per tensor (m_key_shapes / m_value_shapes / m_key_precisions /
+ * m_value_precisions, kv_cache_manager.hpp:74-92) */
+int32_t pa_kv_cache_create_layers(int32_t device, void* stream, const pa_kv_layer_desc* layers, int32_t num_layers,
+                                  pa_kv_cache** out);
 void pa_kv_cache_destroy(pa_kv_cache* cache);
 const char* pa_kv_cache_last_error(const pa_kv_cache* cache);
 /* bytes of one block over all layers, K and V (get_block_size_in_bytes) */

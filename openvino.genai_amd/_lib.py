@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.environ.get("PA_AMD_LIBRARY") or os.path.join(_HERE, "csrc", "libpa_amd.so")
 
 PA_OK = 0
-PA_F16, PA_BF16, PA_U8 = 0, 1, 2
+PA_F16, PA_BF16, PA_U8, PA_U4 = 0, 1, 2, 3
 PA_STATIC_SCRATCH_BYTES = 32 << 20
 PA_AGG_SUM, PA_AGG_NORM_SUM, PA_AGG_ADAPTIVE_RKV = 0, 1, 2
 (PA_KVCRUSH_ANCHOR_RANDOM, PA_KVCRUSH_ANCHOR_ZEROS, PA_KVCRUSH_ANCHOR_ONES, PA_KVCRUSH_ANCHOR_MEAN,
@@ -23,7 +23,7 @@ STATUS_NAMES = {0: "OK", -1: "GENERAL_ERROR", -2: "NOT_IMPLEMENTED", -4: "PARAME
 EXPORTS = [
     "pa_version", "pa_global_last_error", "pa_create", "pa_destroy", "pa_last_error", "pa_step_begin",
     "pa_set_block_indices", "pa_forward", "pa_kv_append", "pa_attention", "pa_attention_static", "pa_synchronize", "pa_get_num_splits", "pa_set_profiling", "pa_last_kernel_ms",
-    "pa_pack_step", "pa_snapkv_num_scores", "pa_kv_cache_create", "pa_kv_cache_destroy", "pa_kv_cache_last_error",
+    "pa_pack_step", "pa_snapkv_num_scores", "pa_kv_cache_create", "pa_kv_cache_create_layers", "pa_kv_cache_destroy", "pa_kv_cache_last_error",
     "pa_kv_cache_block_bytes", "pa_kv_cache_allocate", "pa_kv_cache_num_blocks", "pa_kv_cache_get",
     "pa_kv_cache_copy_blocks", "pa_normalize_num_kv_blocks", "pa_evictor_create", "pa_score_manager_create",
     "pa_evictor_destroy", "pa_evictor_last_error", "pa_evictor_reset_slot", "pa_evictor_register_scores",
@@ -50,7 +50,16 @@ class PaError(RuntimeError):
 class pa_config(C.Structure):
     _fields_ = [("device", C.c_int32), ("num_heads", C.c_int32), ("num_kv_heads", C.c_int32),
                 ("head_size", C.c_int32), ("block_size", C.c_int32), ("query_dtype", C.c_int32),
-                ("kv_cache_dtype", C.c_int32), ("num_layers", C.c_int32), ("stream", C.c_void_p)]
+                ("kv_cache_dtype", C.c_int32), ("num_layers", C.c_int32), ("stream", C.c_void_p),
+                ("v_head_size", C.c_int32), ("value_cache_dtype_p1", C.c_int32)]
+
+
+class pa_kv_tensor_desc(C.Structure):
+    _fields_ = [("num_kv_heads", C.c_int32), ("block_size", C.c_int32), ("head_size", C.c_int32), ("dtype", C.c_int32)]
+
+
+class pa_kv_layer_desc(C.Structure):
+    _fields_ = [("key", pa_kv_tensor_desc), ("value", pa_kv_tensor_desc)]
 
 
 class pa_step_meta(C.Structure):
@@ -112,6 +121,7 @@ def lib():
         "pa_set_rotation_trig_lut": (i32, [vp, P(C.c_float), i32]),
         "pa_rotate_cache": (i32, [vp, vp, i64, P(i32), i32, P(i32), i32]),
         "pa_kv_cache_create": (i32, [P(pa_config), P(vp)]),
+        "pa_kv_cache_create_layers": (i32, [i32, vp, P(pa_kv_layer_desc), i32, P(vp)]),
         "pa_kv_cache_destroy": (None, [vp]),
         "pa_kv_cache_last_error": (C.c_char_p, [vp]),
         "pa_kv_cache_block_bytes": (u64, [vp]),

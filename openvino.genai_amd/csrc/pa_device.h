@@ -6,11 +6,13 @@
 
 namespace pa {
 
-enum : int { DT_F16 = 0, DT_BF16 = 1, DT_U8 = 2 };
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_U8 = 2, DT_U4 = 3 };
 
 constexpr int WAVE = 64;
 
-__host__ __device__ inline int row_bytes(int D, int dt) { return dt == DT_U8 ? D + 8 : D * 2; }
+// bytes of one cached row of D elements: 16-bit values; `f32 scale | f32 zero-point | D codes` (u8); the same header
+// and two codes per byte (u4)
+__host__ __device__ inline int row_bytes(int D, int dt) { return dt == DT_U8 ? D + 8 : dt == DT_U4 ? D / 2 + 8 : D * 2; }
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // ---- 16-bit float bit patterns <-> f32 (device) ----------------------------------------------
@@ -163,12 +165,12 @@ hipError_t launch_kv_append(hipStream_t s, const StepDev& st, const Shape& sh, i
                             const int32_t* block_indices);
 
 // Copy-on-write: block pairs[2 i] -> pairs[2 i + 1] in each of the n_tensors tensors whose base addresses `bases`
-// lists (device arrays); one launch for all of them.
-hipError_t launch_copy_blocks(hipStream_t s, void* const* bases, int n_tensors, const int32_t* pairs, int count,
-                              size_t block_bytes);
+// and block sizes `tensor_block_bytes` list (device arrays); one launch for all of them.
+hipError_t launch_copy_blocks(hipStream_t s, void* const* bases, const uint64_t* tensor_block_bytes, int n_tensors,
+                              const int32_t* pairs, int count, size_t max_block_bytes);
 
 struct AttnWorkspace {
-    float* part_acc;   // [T*Hq*nsplit, D]
+    float* part_acc;   // [T*Hq*nsplit, D] (D: the value head size)
     float* part_ml;    // [T*Hq*nsplit, 2]
     float* final_ml;   // [T*Hq, 2]
     float* logits;     // [Hq, total_scores] raw scaled logits of single-token sequences (scores only)
@@ -176,10 +178,18 @@ struct AttnWorkspace {
     int32_t total_scores;
 };
 
-hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
+// What the shape-generic kernels take: a head size and an element type per cache tensor (query and key rows have Dk
+// elements, value and output rows Dv; both multiples of 8, at most GENERIC_MAX_HEAD_SIZE).
+constexpr int GENERIC_MAX_HEAD_SIZE = 512;
+struct GenericShape {
+    int32_t Hq, Hkv, Dk, Dv, bs, kdt, vdt;
+};
+hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype,
                                     const void* query, const void* key_cache, const void* value_cache,
                                     const int32_t* block_indices, const AttnWorkspace& ws, void* out, float* scores,
                                     int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1);
+hipError_t launch_kv_append_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype, const void* key,
+                                    const void* value, void* key_cache, void* value_cache, const int32_t* block_indices);
 
 // What a workgroup of the u8 decode kernel needs to start fetching KV blocks, resolved on the host when the block
 // table is set: one entry per (listed sequence, split), read with one scalar load instead of a chain of dependent

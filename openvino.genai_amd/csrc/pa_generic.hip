@@ -1,71 +1,90 @@
-// Shape-generic PagedAttention kernels (any block size, GQA ratio, head size 64/128, q_len >= 1).
+// Shape-generic PagedAttention kernels: any block size and GQA ratio, q_len >= 1, key and value head sizes that are
+// multiples of 8 up to 512 and need not be equal, and an element type per cache tensor -- f16, bf16, u8 rows
+// (`f32 scale | f32 zero-point | D codes`) or u4 rows (`f32 scale | f32 zero-point | D / 2 bytes`, element 2 i in the
+// high nibble of byte i).  Everything the tuned kernels do not take runs here.
 //
-// pa_generic_kernel : one wave per (token, query head, split).  Lanes take consecutive KV positions
-//                     for QK (each lane owns one cache row), then the wave walks the 64 positions
-//                     with lanes across the head dimension for PV.  Online softmax per wave.
-// pa_merge_kernel   : folds the split partials (m, l, acc) into the output row and keeps the final
-//                     (max, denominator) of every (token, head) for the score kernels.
-// pa_scores_single  : scores of single-token (decode) sequences from the stored logits.
-// pa_scores_window  : scores of multi-token sequences: recomputes QK for the last W query rows.
+// pa_generic_kernel     : one wave per (token, query head, split).  Lanes take consecutive KV positions for QK (each
+//                         lane owns one cache row), then the wave walks the 64 positions with lanes across the value
+//                         head for PV.  Online softmax per wave.
+// pa_merge_kernel       : folds the split partials (m, l, acc) into the output row and keeps the final
+//                         (max, denominator) of every (token, head) for the score kernels.
+// pa_scores_single      : scores of single-token (decode) sequences from the stored logits.
+// pa_scores_window      : scores of multi-token sequences: recomputes QK for the last W query rows.
+// kv_append_generic     : one wave per (token, kv head, K | V) row: copy / convert / quantise into the cache row.
 //
-// These are the fallback for shapes the tuned kernels do not cover; HBM-bound, no MFMA.
+// HBM-bound, no MFMA: a fallback, not a tuned path.
 #include "pa_device.h"
 
 namespace pa {
 namespace {
 
-// Dequantised element pair access --------------------------------------------------------------
-template <int KVDT>
+constexpr int MAX_D = GENERIC_MAX_HEAD_SIZE;
+
+// One cached row of D elements in the tensor's element type, read as f32.
 struct RowReader {
     const uint8_t* row;
     float scale, zp;
-    __device__ RowReader(const uint8_t* cache, long phys, int h, int slot, const Shape& sh) {
-        row = cache + ((phys * sh.Hkv + h) * sh.bs + slot) * (long)row_bytes(sh.D, KVDT);
-        if (KVDT == DT_U8) {
-            float2 hdr = *reinterpret_cast<const float2*>(row);
+    int dt;
+    __device__ RowReader(const uint8_t* cache, long phys, int h, int slot, int Hkv, int bs, int D, int dt_) : dt(dt_) {
+        row = cache + ((phys * Hkv + h) * bs + slot) * (long)row_bytes(D, dt_);
+        scale = 1.0f;
+        zp = 0.0f;
+        if (dt == DT_U8 || dt == DT_U4) {
+            const float2 hdr = *reinterpret_cast<const float2*>(row);
             scale = hdr.x;
             zp = hdr.y;
             row += 8;
-        } else {
-            scale = 1.0f;
-            zp = 0.0f;
         }
     }
     // eight consecutive elements starting at d (d % 8 == 0)
     __device__ void load8(int d, float* out) const {
-        if (KVDT == DT_U8) {
-            uint2 v = *reinterpret_cast<const uint2*>(row + d);
+        if (dt == DT_U8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(row + d);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 out[e] = ((float)((v.x >> (8 * e)) & 0xff) - zp) * scale;
                 out[4 + e] = ((float)((v.y >> (8 * e)) & 0xff) - zp) * scale;
             }
+        } else if (dt == DT_U4) {
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(row + d / 2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {  // byte e holds elements 2 e (high nibble) and 2 e + 1 (low nibble)
+                const uint32_t byte = (v >> (8 * e)) & 0xff;
+                out[2 * e] = ((float)(byte >> 4) - zp) * scale;
+                out[2 * e + 1] = ((float)(byte & 15) - zp) * scale;
+            }
         } else {
-            uint4 v = *reinterpret_cast<const uint4*>(row + 2 * d);
+            const uint4 v = *reinterpret_cast<const uint4*>(row + 2 * d);
             const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                out[2 * e] = load16<KVDT == DT_U8 ? DT_F16 : KVDT>((uint16_t)(w[e] & 0xffff));
-                out[2 * e + 1] = load16<KVDT == DT_U8 ? DT_F16 : KVDT>((uint16_t)(w[e] >> 16));
+                out[2 * e] = dt == DT_F16 ? half_bits_to_float((uint16_t)(w[e] & 0xffff)) : bf16_bits_to_float((uint16_t)(w[e] & 0xffff));
+                out[2 * e + 1] = dt == DT_F16 ? half_bits_to_float((uint16_t)(w[e] >> 16)) : bf16_bits_to_float((uint16_t)(w[e] >> 16));
             }
         }
     }
     __device__ float load1(int d) const {
-        if (KVDT == DT_U8) return ((float)row[d] - zp) * scale;
-        return load16<KVDT == DT_U8 ? DT_F16 : KVDT>(reinterpret_cast<const uint16_t*>(row)[d]);
+        if (dt == DT_U8) return ((float)row[d] - zp) * scale;
+        if (dt == DT_U4) {
+            const uint8_t byte = row[d >> 1];
+            return ((float)((d & 1) ? (byte & 15) : (byte >> 4)) - zp) * scale;
+        }
+        const uint16_t v = reinterpret_cast<const uint16_t*>(row)[d];
+        return dt == DT_F16 ? half_bits_to_float(v) : bf16_bits_to_float(v);
     }
 };
 
-template <int D, int QDT, int KVDT>
-__global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ query,
+template <int QDT>
+__global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, GenericShape sh, const uint16_t* __restrict__ query,
                                                          const uint8_t* __restrict__ key_cache,
                                                          const uint8_t* __restrict__ value_cache,
                                                          const int32_t* __restrict__ block_indices, AttnWorkspace ws,
                                                          int store_logits) {
-    constexpr int EPL = D / 64;
-    __shared__ float qs[4][D];
+    constexpr int EPL = MAX_D / 64;  // value channels per lane at most
+    __shared__ float qs[4][MAX_D];
     const int lane = threadIdx.x & 63;
     const int wv = threadIdx.x >> 6;
+    const int Dk = sh.Dk, Dv = sh.Dv;
     const long wave = (long)blockIdx.x * 4 + wv;
     const long total = (long)st.T * sh.Hq * ws.nsplit;
     const bool valid = wave < total;
@@ -74,7 +93,7 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, Shape sh, c
         split = (int)(wave % ws.nsplit);
         hq = (int)((wave / ws.nsplit) % sh.Hq);
         t = (int)(wave / ((long)ws.nsplit * sh.Hq));
-        for (int d = lane; d < D; d += 64) qs[wv][d] = load16<QDT>(query[((long)t * sh.Hq + hq) * D + d]) * st.scale;
+        for (int d = lane; d < Dk; d += 64) qs[wv][d] = load16<QDT>(query[((long)t * sh.Hq + hq) * Dk + d]) * st.scale;
     }
     __syncthreads();
     if (!valid) return;
@@ -106,10 +125,9 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, Shape sh, c
         float s = -INFINITY;
         if (live) {
             phys = table[j / sh.bs];
-            RowReader<KVDT> kr(key_cache, phys, hkv, j % sh.bs, sh);
+            RowReader kr(key_cache, phys, hkv, j % sh.bs, sh.Hkv, sh.bs, Dk, sh.kdt);
             float dot = 0.0f;
-#pragma unroll 4
-            for (int d = 0; d < D; d += 8) {
+            for (int d = 0; d < Dk; d += 8) {
                 float k8[8];
                 kr.load8(d, k8);
 #pragma unroll
@@ -129,9 +147,10 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, Shape sh, c
         for (int jj = 0; jj < cnt; ++jj) {
             const float pj = __shfl(p, jj, WAVE);
             const long pb = __shfl(phys, jj, WAVE);
-            RowReader<KVDT> vr(value_cache, pb, hkv, (j0 + jj) % sh.bs, sh);
+            RowReader vr(value_cache, pb, hkv, (j0 + jj) % sh.bs, sh.Hkv, sh.bs, Dv, sh.vdt);
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[e] += pj * vr.load1(lane * EPL + e);
+            for (int e = 0; e < EPL; ++e)
+                if (lane + 64 * e < Dv) acc[e] += pj * vr.load1(lane + 64 * e);
         }
     }
     const long slot = ((long)t * sh.Hq + hq) * ws.nsplit + split;
@@ -140,13 +159,15 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, Shape sh, c
         ws.part_ml[2 * slot + 1] = l;
     }
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) ws.part_acc[slot * D + lane * EPL + e] = acc[e];
+    for (int e = 0; e < EPL; ++e)
+        if (lane + 64 * e < Dv) ws.part_acc[slot * Dv + lane + 64 * e] = acc[e];
 }
 
-template <int D, int QDT>
-__global__ __launch_bounds__(256) void pa_merge_kernel(StepDev st, Shape sh, AttnWorkspace ws, uint16_t* __restrict__ out) {
-    constexpr int EPL = D / 64;
+template <int QDT>
+__global__ __launch_bounds__(256) void pa_merge_kernel(StepDev st, GenericShape sh, AttnWorkspace ws, uint16_t* __restrict__ out) {
+    constexpr int EPL = MAX_D / 64;
     const int lane = threadIdx.x & 63;
+    const int Dv = sh.Dv;
     const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= (long)st.T * sh.Hq) return;
     float M = -INFINITY;
@@ -162,11 +183,13 @@ __global__ __launch_bounds__(256) void pa_merge_kernel(StepDev st, Shape sh, Att
         const float f = __expf(ms - M);
         L += ws.part_ml[2 * slot + 1] * f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] += ws.part_acc[slot * D + lane * EPL + e] * f;
+        for (int e = 0; e < EPL; ++e)
+            if (lane + 64 * e < Dv) acc[e] += ws.part_acc[slot * Dv + lane + 64 * e] * f;
     }
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) out[row * D + lane * EPL + e] = store16<QDT>(acc[e] * inv);
+    for (int e = 0; e < EPL; ++e)
+        if (lane + 64 * e < Dv) out[row * Dv + lane + 64 * e] = store16<QDT>(acc[e] * inv);
     if (lane == 0) {
         ws.final_ml[2 * row] = M;
         ws.final_ml[2 * row + 1] = L;
@@ -174,7 +197,7 @@ __global__ __launch_bounds__(256) void pa_merge_kernel(StepDev st, Shape sh, Att
 }
 
 // Single-token sequences: score_j = sum over heads of exp(logit - M) / L, heads in ascending order.
-__global__ __launch_bounds__(256) void pa_scores_single_kernel(StepDev st, Shape sh, AttnWorkspace ws,
+__global__ __launch_bounds__(256) void pa_scores_single_kernel(StepDev st, GenericShape sh, AttnWorkspace ws,
                                                                float* __restrict__ scores) {
     const int b = blockIdx.y;
     const int q_len = st.subsequence_begins[b + 1] - st.subsequence_begins[b];
@@ -197,8 +220,8 @@ __global__ __launch_bounds__(256) void pa_scores_single_kernel(StepDev st, Shape
 }
 
 // Multi-token sequences: the last W query rows are replayed against every position they can see.
-template <int D, int QDT, int KVDT>
-__global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, Shape sh, AttnWorkspace ws,
+template <int QDT>
+__global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, GenericShape sh, AttnWorkspace ws,
                                                                const uint16_t* __restrict__ query,
                                                                const uint8_t* __restrict__ key_cache,
                                                                const int32_t* __restrict__ block_indices,
@@ -211,6 +234,7 @@ __global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, Shape
     const int kv_len = past + q_len;
     const int W = st.score_window[b];
     const int G = sh.Hq / sh.Hkv;
+    const int Dk = sh.Dk;
     const int32_t* table = block_indices + st.block_indices_begins[b];
     for (int j = blockIdx.x * 256 + threadIdx.x; j < kv_len; j += gridDim.x * 256) {
         float sum = 0.0f;
@@ -219,13 +243,13 @@ __global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, Shape
             const int first = st.sliding_window > 0 ? max(0, last + 1 - st.sliding_window) : 0;
             if (j < first || j > last) continue;
             for (int h = 0; h < sh.Hq; ++h) {
-                RowReader<KVDT> kr(key_cache, table[j / sh.bs], h / G, j % sh.bs, sh);
-                const uint16_t* q = query + ((long)(t0 + i) * sh.Hq + h) * D;
+                RowReader kr(key_cache, table[j / sh.bs], h / G, j % sh.bs, sh.Hkv, sh.bs, Dk, sh.kdt);
+                const uint16_t* q = query + ((long)(t0 + i) * sh.Hq + h) * Dk;
                 float dot = 0.0f;
-                for (int d = 0; d < D; d += 8) {
+                for (int d = 0; d < Dk; d += 8) {
                     float k8[8];
                     kr.load8(d, k8);
-                    uint4 qv = *reinterpret_cast<const uint4*>(q + d);
+                    const uint4 qv = *reinterpret_cast<const uint4*>(q + d);
                     const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -242,8 +266,78 @@ __global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, Shape
     }
 }
 
-template <int D, int QDT, int KVDT>
-hipError_t launch_typed(hipStream_t s, const StepDev& st, const Shape& sh, const void* query, const void* kc,
+// One wave per (token, kv head, K | V) row.  u8 / u4 rows: scale = (max - min) / levels (a zero range takes 1e-4),
+// zp = -min / scale, code = clamp(rne(fma(x, 1 / scale, zp)), 0, levels), every operation in IEEE binary32 without
+// contraction, so that the bytes are reproducible on any IEEE host.  16-bit rows are copied, or converted when the cache
+// holds the other 16-bit type.
+template <int QDT>
+__global__ __launch_bounds__(256) void kv_append_generic_kernel(StepDev st, GenericShape sh, const uint16_t* __restrict__ key,
+                                                                const uint16_t* __restrict__ value,
+                                                                uint8_t* __restrict__ key_cache,
+                                                                uint8_t* __restrict__ value_cache,
+                                                                const int32_t* __restrict__ block_indices) {
+#pragma clang fp contract(off)
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (long)st.T * sh.Hkv * 2) return;
+    const int which = (int)(row & 1);
+    const int h = (int)((row >> 1) % sh.Hkv);
+    const int t = (int)((row >> 1) / sh.Hkv);
+    const int D = which ? sh.Dv : sh.Dk, dt = which ? sh.vdt : sh.kdt;
+    const int b = st.token_seq[t];
+    const int slot = st.past_lens[b] + t - st.subsequence_begins[b];
+    const long phys = block_indices[st.block_indices_begins[b] + slot / sh.bs];
+    const uint16_t* src = (which ? value : key) + ((long)t * sh.Hkv + h) * D;
+    uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)row_bytes(D, dt);
+    constexpr int PPL = MAX_D / 128;  // element pairs per lane at most
+    float x0[PPL], x1[PPL];
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PPL; ++i) {
+        const int p = lane + 64 * i;
+        if (2 * p < D) {
+            const uint32_t w = reinterpret_cast<const uint32_t*>(src)[p];
+            x0[i] = load16<QDT>((uint16_t)(w & 0xffff));
+            x1[i] = load16<QDT>((uint16_t)(w >> 16));
+            mn = fminf(mn, fminf(x0[i], x1[i]));
+            mx = fmaxf(mx, fmaxf(x0[i], x1[i]));
+        }
+    }
+    if (dt == DT_F16 || dt == DT_BF16) {
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) {
+            const int p = lane + 64 * i;
+            if (2 * p < D) {
+                const uint32_t lo = dt == DT_F16 ? float_to_half_bits(x0[i]) : float_to_bf16_bits(x0[i]);
+                const uint32_t hi = dt == DT_F16 ? float_to_half_bits(x1[i]) : float_to_bf16_bits(x1[i]);
+                // (the cache's own type: the bits as they came; the other 16-bit type: converted)
+                reinterpret_cast<uint32_t*>(dst)[p] = dt == QDT ? reinterpret_cast<const uint32_t*>(src)[p] : (lo | (hi << 16));
+            }
+        }
+        return;
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    const float levels = dt == DT_U8 ? 255.0f : 15.0f;
+    float scale = (mx - mn) / levels;
+    if (scale == 0.0f) scale = 0.0001f;
+    const float zp = -mn / scale;
+    const float inv = 1.0f / scale;
+    if (lane == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
+#pragma unroll
+    for (int i = 0; i < PPL; ++i) {
+        const int p = lane + 64 * i;
+        if (2 * p < D) {
+            const float c0 = fminf(fmaxf(rintf(__fmaf_rn(x0[i], inv, zp)), 0.0f), levels);
+            const float c1 = fminf(fmaxf(rintf(__fmaf_rn(x1[i], inv, zp)), 0.0f), levels);
+            if (dt == DT_U8) reinterpret_cast<uint16_t*>(dst + 8)[p] = (uint16_t)((uint32_t)(int)c0 | ((uint32_t)(int)c1 << 8));
+            else dst[8 + p] = (uint8_t)(((uint32_t)(int)c0 << 4) | (uint32_t)(int)c1);
+        }
+    }
+}
+
+template <int QDT>
+hipError_t launch_typed(hipStream_t s, const StepDev& st, const GenericShape& sh, const void* query, const void* kc,
                         const void* vc, const int32_t* bi, const AttnWorkspace& ws, void* out, float* scores,
                         int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1) {
     const long waves = (long)st.T * sh.Hq * ws.nsplit;
@@ -252,50 +346,55 @@ hipError_t launch_typed(hipStream_t s, const StepDev& st, const Shape& sh, const
     auto k = reinterpret_cast<const uint8_t*>(kc);
     auto v = reinterpret_cast<const uint8_t*>(vc);
     if (ev0) (void)hipEventRecord(ev0, s);
-    hipLaunchKernelGGL((pa_generic_kernel<D, QDT, KVDT>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, st, sh, q,
-                       k, v, bi, ws, scores ? 1 : 0);
+    hipLaunchKernelGGL((pa_generic_kernel<QDT>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, st, sh, q, k, v, bi, ws,
+                       scores ? 1 : 0);
     if (ev1) (void)hipEventRecord(ev1, s);
     const long rows = (long)st.T * sh.Hq;
-    hipLaunchKernelGGL((pa_merge_kernel<D, QDT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, st, sh, ws,
+    hipLaunchKernelGGL((pa_merge_kernel<QDT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, st, sh, ws,
                        reinterpret_cast<uint16_t*>(out));
     if (scores) {
         dim3 grid((unsigned)min(ceil_div(max_kv_len, 256), 1024), (unsigned)st.B);
         hipLaunchKernelGGL(pa_scores_single_kernel, grid, dim3(256), 0, s, st, sh, ws, scores);
         if (st.T > st.B)
-            hipLaunchKernelGGL((pa_scores_window_kernel<D, QDT, KVDT>), grid, dim3(256), 0, s, st, sh, ws, q, k, bi,
-                               scores, 0);
+            hipLaunchKernelGGL((pa_scores_window_kernel<QDT>), grid, dim3(256), 0, s, st, sh, ws, q, k, bi, scores, 0);
     }
     return hipGetLastError();
 }
 
-template <int D>
-hipError_t launch_d(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype, const void* query,
-                    const void* kc, const void* vc, const int32_t* bi, const AttnWorkspace& ws, void* out,
-                    float* scores, int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1) {
-#define PA_CASE(Q, K)                                                                                               \
-    if (q_dtype == Q && kv_dtype == K)                                                                              \
-        return launch_typed<D, Q, K>(s, st, sh, query, kc, vc, bi, ws, out, scores, max_kv_len, ev0, ev1);
-    PA_CASE(DT_F16, DT_F16)
-    PA_CASE(DT_F16, DT_BF16)
-    PA_CASE(DT_F16, DT_U8)
-    PA_CASE(DT_BF16, DT_F16)
-    PA_CASE(DT_BF16, DT_BF16)
-    PA_CASE(DT_BF16, DT_U8)
-#undef PA_CASE
-    return hipErrorInvalidValue;
+bool generic_shape_ok(const GenericShape& sh) {
+    auto dt_ok = [](int dt) { return dt == DT_F16 || dt == DT_BF16 || dt == DT_U8 || dt == DT_U4; };
+    return sh.Dk > 0 && sh.Dv > 0 && sh.Dk % 8 == 0 && sh.Dv % 8 == 0 && sh.Dk <= MAX_D && sh.Dv <= MAX_D && dt_ok(sh.kdt) &&
+           dt_ok(sh.vdt);
 }
 
 }  // namespace
 
-hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const Shape& sh, int q_dtype, int kv_dtype,
+hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype,
                                     const void* query, const void* key_cache, const void* value_cache,
                                     const int32_t* block_indices, const AttnWorkspace& ws, void* out, float* scores,
                                     int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1) {
-    if (sh.D == 64)
-        return launch_d<64>(s, st, sh, q_dtype, kv_dtype, query, key_cache, value_cache, block_indices, ws, out, scores, max_kv_len, ev0, ev1);
-    if (sh.D == 128)
-        return launch_d<128>(s, st, sh, q_dtype, kv_dtype, query, key_cache, value_cache, block_indices, ws, out, scores, max_kv_len, ev0, ev1);
+    if (!generic_shape_ok(sh)) return hipErrorInvalidValue;
+    if (q_dtype == DT_F16)
+        return launch_typed<DT_F16>(s, st, sh, query, key_cache, value_cache, block_indices, ws, out, scores, max_kv_len, ev0, ev1);
+    if (q_dtype == DT_BF16)
+        return launch_typed<DT_BF16>(s, st, sh, query, key_cache, value_cache, block_indices, ws, out, scores, max_kv_len, ev0, ev1);
     return hipErrorInvalidValue;
+}
+
+hipError_t launch_kv_append_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype, const void* key,
+                                    const void* value, void* key_cache, void* value_cache, const int32_t* block_indices) {
+    if (!generic_shape_ok(sh)) return hipErrorInvalidValue;
+    const long rows = (long)st.T * sh.Hkv * 2;
+    if (rows == 0) return hipSuccess;
+    auto k = reinterpret_cast<const uint16_t*>(key);
+    auto v = reinterpret_cast<const uint16_t*>(value);
+    auto kc = reinterpret_cast<uint8_t*>(key_cache);
+    auto vc = reinterpret_cast<uint8_t*>(value_cache);
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    if (q_dtype == DT_F16) hipLaunchKernelGGL((kv_append_generic_kernel<DT_F16>), grid, dim3(256), 0, s, st, sh, k, v, kc, vc, block_indices);
+    else if (q_dtype == DT_BF16) hipLaunchKernelGGL((kv_append_generic_kernel<DT_BF16>), grid, dim3(256), 0, s, st, sh, k, v, kc, vc, block_indices);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 }  // namespace pa

@@ -86,16 +86,29 @@ void check_config(const pa_config* c) {
     PA_REQUIRE(c, PA_INVALID_C_PARAM, "config is null");
     PA_REQUIRE(c->num_heads > 0 && c->num_kv_heads > 0 && c->num_heads % c->num_kv_heads == 0, PA_PARAMETER_MISMATCH,
                "num_heads must be a positive multiple of num_kv_heads");
-    PA_REQUIRE(c->head_size == 64 || c->head_size == 128, PA_NOT_IMPLEMENTED, "head_size must be 64 or 128");
+    auto head_ok = [](int32_t d) { return d >= 8 && d <= pa::GENERIC_MAX_HEAD_SIZE && d % 8 == 0; };
+    auto cache_dt_ok = [](int32_t dt) { return dt == PA_F16 || dt == PA_BF16 || dt == PA_U8 || dt == PA_U4; };
+    PA_REQUIRE(head_ok(c->head_size), PA_NOT_IMPLEMENTED, "head_size must be a multiple of 8 between 8 and 512");
+    PA_REQUIRE(c->v_head_size == 0 || head_ok(c->v_head_size), PA_NOT_IMPLEMENTED,
+               "v_head_size must be 0 (= head_size) or a multiple of 8 between 8 and 512");
     PA_REQUIRE(c->block_size > 0, PA_PARAMETER_MISMATCH, "block_size must be positive");
     PA_REQUIRE(c->query_dtype == PA_F16 || c->query_dtype == PA_BF16, PA_PARAMETER_MISMATCH,
                "query_dtype must be PA_F16 or PA_BF16");
-    PA_REQUIRE(c->kv_cache_dtype == PA_F16 || c->kv_cache_dtype == PA_BF16 || c->kv_cache_dtype == PA_U8,
-               PA_PARAMETER_MISMATCH, "kv_cache_dtype must be PA_U8, PA_F16 or PA_BF16");
+    PA_REQUIRE(cache_dt_ok(c->kv_cache_dtype), PA_PARAMETER_MISMATCH, "kv_cache_dtype must be PA_U8, PA_U4, PA_F16 or PA_BF16");
+    PA_REQUIRE(c->value_cache_dtype_p1 == 0 || cache_dt_ok(c->value_cache_dtype_p1 - 1), PA_PARAMETER_MISMATCH,
+               "value_cache_dtype_p1 must be 0 (= kv_cache_dtype) or 1 + PA_U8 / PA_U4 / PA_F16 / PA_BF16");
     PA_REQUIRE(c->num_layers > 0, PA_PARAMETER_MISMATCH, "num_layers must be positive");
     int ndev = 0;
     HIP_CHECK(hipGetDeviceCount(&ndev));
     PA_REQUIRE(c->device >= 0 && c->device < ndev, PA_OUT_OF_BOUNDS, "no such HIP device");
+}
+
+// The value side of a configuration (0 in either field = as the key side).
+int32_t v_head(const pa_config& c) { return c.v_head_size ? c.v_head_size : c.head_size; }
+int32_t v_dtype(const pa_config& c) { return c.value_cache_dtype_p1 ? c.value_cache_dtype_p1 - 1 : c.kv_cache_dtype; }
+// K and V alike, in a type the tuned kernels read (they also want head size 64 or 128: checked where they are chosen)
+bool kv_alike(const pa_config& c) {
+    return v_head(c) == c.head_size && v_dtype(c) == c.kv_cache_dtype && c.kv_cache_dtype != PA_U4;
 }
 
 // Fixed device scratch of pa_attention_static: one copy per GPU the library runs on, held until the process ends.
@@ -196,16 +209,20 @@ struct pa_kv_cache {
     uint64_t num_blocks = 0;
     std::vector<void*> key, value;      // base addresses (fixed from creation on)
     size_t granularity = 0;             // size of every physical piece: memory is mapped in equal, equally aligned pieces
-    size_t reserved = 0, mapped = 0;    // per tensor: bytes of address space / bytes backed by memory
+    // per tensor (2 * layer + (0 = K, 1 = V)): bytes of one block, of address space, and of address space backed by memory
+    std::vector<uint64_t> block_bytes;
+    std::vector<size_t> reserved, mapped;
     struct Chunk {
         hipMemGenericAllocationHandle_t handle;
         size_t offset, bytes;
     };
-    std::vector<std::vector<Chunk>> chunks;  // per tensor: 2 * layer + (0 = K, 1 = V)
-    DevBuf base_table;                  // the 2 * num_layers base addresses, for the copy kernel
+    std::vector<std::vector<Chunk>> chunks;  // per tensor
+    DevBuf base_table;                  // the 2 * num_layers base addresses, then the tensors' block sizes, for the copy kernel
     DevBuf pairs;                       // (source, destination) list of one copy launch
-    uint64_t layer_block_bytes() const {  // one block of K (or V) in one layer
-        return (uint64_t)cfg.num_kv_heads * cfg.block_size * pa::row_bytes(cfg.head_size, cfg.kv_cache_dtype);
+    uint64_t all_block_bytes() const {  // one block over every tensor
+        uint64_t sum = 0;
+        for (uint64_t b : block_bytes) sum += b;
+        return sum;
     }
     void*& tensor(size_t t) { return (t & 1) ? value[t >> 1] : key[t >> 1]; }
 };
@@ -236,6 +253,12 @@ int32_t guarded(Obj* obj, Fn&& fn) {
 struct NoObj { std::string error; };
 
 pa::Shape shape_of(const pa_config& c) { return pa::Shape{c.num_heads, c.num_kv_heads, c.head_size, c.block_size}; }
+pa::GenericShape generic_shape_of(const pa_config& c) {
+    return pa::GenericShape{c.num_heads, c.num_kv_heads, c.head_size, v_head(c), c.block_size, c.kv_cache_dtype, v_dtype(c)};
+}
+// The append kernel with a row per 16 lanes is built for K and V alike, head size 64 or 128; everything else takes the
+// shape-generic one (a wave per row).
+bool tuned_append_shape(const pa_config& c) { return kv_alike(c) && (c.head_size == 64 || c.head_size == 128); }
 
 const int32_t* table_for(pa_ctx* ctx, int32_t layer) {
     PA_REQUIRE(layer >= 0 && layer < ctx->cfg.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
@@ -299,8 +322,12 @@ void fill_decode_descs(const pa_ctx* ctx, const int32_t* ids, uint8_t* stage) {
 void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
     check_io(ctx, layer, io, true, false);
     const int32_t* table = table_for(ctx, layer);
-    HIP_CHECK(pa::launch_kv_append(ctx->stream, ctx->dev, shape_of(ctx->cfg), ctx->cfg.query_dtype,
-                                   ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
+    if (tuned_append_shape(ctx->cfg))
+        HIP_CHECK(pa::launch_kv_append(ctx->stream, ctx->dev, shape_of(ctx->cfg), ctx->cfg.query_dtype,
+                                       ctx->cfg.kv_cache_dtype, io->key, io->value, io->key_cache, io->value_cache, table));
+    else
+        HIP_CHECK(pa::launch_kv_append_generic(ctx->stream, ctx->dev, generic_shape_of(ctx->cfg), ctx->cfg.query_dtype,
+                                               io->key, io->value, io->key_cache, io->value_cache, table));
 }
 
 // Block sizes the tuned kernels take.  Their tiles are 32 tokens: two 16-token cache blocks, one 32-token block, or a
@@ -309,20 +336,20 @@ bool tuned_block_size(int32_t bs) { return bs >= 16 && bs <= 256 && (bs & (bs - 
 
 // Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).
 bool decode_u8_shape(const pa_config& c) {
-    return c.kv_cache_dtype == PA_U8 && tuned_block_size(c.block_size) &&
+    return kv_alike(c) && c.kv_cache_dtype == PA_U8 && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
 bool mfma_shape(const pa_config& c) {
-    return (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && tuned_block_size(c.block_size) &&
+    return kv_alike(c) && (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 256;
 }
 
 // Shapes the 16-bit decode kernel is built for (single-token sequences of a call that asks for no scores).
 bool decode16_shape(const pa_config& c) {
-    return c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && tuned_block_size(c.block_size) &&
+    return kv_alike(c) && c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
 
@@ -884,13 +911,13 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;
-    ctx->part_acc.reserve(rows * ctx->nsplit * c.head_size * sizeof(float));
+    ctx->part_acc.reserve(rows * ctx->nsplit * v_head(c) * sizeof(float));
     ctx->part_ml.reserve(rows * ctx->nsplit * 2 * sizeof(float));
     ctx->final_ml.reserve(rows * 2 * sizeof(float));
     if (io->scores) ctx->logits.reserve((size_t)c.num_heads * ctx->total_scores * sizeof(float));
     pa::AttnWorkspace ws{ctx->part_acc.as<float>(), ctx->part_ml.as<float>(), ctx->final_ml.as<float>(),
                          ctx->logits.as<float>(), ctx->nsplit, ctx->total_scores};
-    HIP_CHECK(pa::launch_attention_generic(ctx->stream, ctx->dev, shape_of(c), c.query_dtype, c.kv_cache_dtype,
+    HIP_CHECK(pa::launch_attention_generic(ctx->stream, ctx->dev, generic_shape_of(c), c.query_dtype,
                                            io->query, io->key_cache, io->value_cache, table, ws, io->out, io->scores,
                                            ctx->max_kv, ctx->profiling ? ctx->ev0 : nullptr,
                                            ctx->profiling ? ctx->ev1 : nullptr));
@@ -1427,6 +1454,7 @@ int32_t pa_rotate_cache(pa_ctx* ctx, void* key_cache, int64_t num_blocks, const 
         if (num_rotated == 0) return;
         PA_REQUIRE(key_cache && rotated_block_indices && rotation_deltas, PA_INVALID_C_PARAM, "null argument");
         PA_REQUIRE(ctx->trig_rows > 0, PA_NOT_ALLOCATED, "pa_set_rotation_trig_lut has not been called");
+        PA_REQUIRE(c.kv_cache_dtype != PA_U4, PA_NOT_IMPLEMENTED, "cache rotation runs over u8, f16 and bf16 key caches");
         PA_REQUIRE(deltas_per_block == 1 || deltas_per_block == c.block_size, PA_PARAMETER_MISMATCH,
                    "rotation_deltas must hold 1 or block_size entries per block");
         for (int32_t i = 0; i < num_rotated; ++i)
@@ -1458,8 +1486,8 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         PA_REQUIRE(ctx->step_ready, PA_PARAMETER_MISMATCH, "pa_step_begin has not been called");
         PA_REQUIRE(evictable_sizes, PA_INVALID_C_PARAM, "adaptive_rkv_evictable_sizes missing");
         PA_REQUIRE(layer >= 0 && layer < c.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
-        PA_REQUIRE(c.block_size == 32 && (c.head_size == 64 || c.head_size == 128), PA_NOT_IMPLEMENTED,
-                   "block diversity runs for block size 32 and head size 64 or 128");
+        PA_REQUIRE(c.block_size == 32 && (c.head_size == 64 || c.head_size == 128) && c.kv_cache_dtype != PA_U4, PA_NOT_IMPLEMENTED,
+                   "block diversity runs for block size 32, head size 64 or 128 and a u8, f16 or bf16 key cache");
         PA_REQUIRE(start_size >= 0 && start_size % c.block_size == 0, PA_PARAMETER_MISMATCH,
                    "adaptive_rkv_start_size must be a non-negative multiple of the block size");
         const size_t tidx = ctx->shared_table ? 0 : (size_t)layer;
@@ -1584,7 +1612,7 @@ void destroy_kv_cache(pa_kv_cache* c) {
     (void)hipDeviceSynchronize();
     drop_chunks(c, std::vector<size_t>(c->chunks.size(), 0));
     for (size_t t = 0; t < 2 * c->key.size(); ++t)
-        if (c->tensor(t)) (void)hipMemAddressFree(c->tensor(t), c->reserved);
+        if (c->tensor(t)) (void)hipMemAddressFree(c->tensor(t), c->reserved[t]);
     c->base_table.release();
     c->pairs.release();
     delete c;
@@ -1592,49 +1620,93 @@ void destroy_kv_cache(pa_kv_cache* c) {
 
 }  // namespace
 
+namespace {
+// The tensors of a cache from one description per layer (key and value side of each).
+void create_kv_cache(int32_t device, void* stream, const pa_kv_layer_desc* layers, int32_t num_layers, pa_kv_cache** out) {
+    PA_REQUIRE(out, PA_INVALID_C_PARAM, "out is null");
+    *out = nullptr;
+    PA_REQUIRE(layers && num_layers > 0, PA_INVALID_C_PARAM, "layer descriptions missing");
+    int ndev = 0;
+    HIP_CHECK(hipGetDeviceCount(&ndev));
+    PA_REQUIRE(device >= 0 && device < ndev, PA_OUT_OF_BOUNDS, "no such HIP device");
+    HIP_CHECK(hipSetDevice(device));
+    pa_kv_cache* c = new pa_kv_cache();
+    c->cfg.device = device;
+    c->cfg.stream = stream;
+    c->cfg.num_layers = num_layers;
+    const size_t n_tensors = 2 * (size_t)num_layers;
+    c->key.assign(num_layers, nullptr);
+    c->value.assign(num_layers, nullptr);
+    c->chunks.assign(n_tensors, {});
+    c->block_bytes.assign(n_tensors, 0);
+    c->reserved.assign(n_tensors, 0);
+    c->mapped.assign(n_tensors, 0);
+    try {
+        for (size_t t = 0; t < n_tensors; ++t) {
+            const pa_kv_tensor_desc& d = (t & 1) ? layers[t >> 1].value : layers[t >> 1].key;
+            PA_REQUIRE(d.num_kv_heads > 0 && d.block_size > 0 && d.head_size > 0, PA_PARAMETER_MISMATCH,
+                       "kv heads, block size and head size of a cache tensor must be positive");
+            PA_REQUIRE(d.dtype == PA_F16 || d.dtype == PA_BF16 || d.dtype == PA_U8 || d.dtype == PA_U4, PA_PARAMETER_MISMATCH,
+                       "a cache tensor's type must be PA_U8, PA_U4, PA_F16 or PA_BF16");
+            PA_REQUIRE(d.dtype != PA_U4 || d.head_size % 2 == 0, PA_PARAMETER_MISMATCH, "u4 rows hold an even number of elements");
+            c->block_bytes[t] = (uint64_t)d.num_kv_heads * d.block_size * pa::row_bytes(d.head_size, d.dtype);
+            PA_REQUIRE(c->block_bytes[t] % 16 == 0, PA_NOT_IMPLEMENTED, "a block of one tensor must be a multiple of 16 bytes");
+        }
+        const hipMemAllocationProp prop = device_memory_prop(device);
+        size_t reported = 0;
+        HIP_CHECK(hipMemGetAllocationGranularity(&reported, &prop, hipMemAllocationGranularityRecommended));
+        PA_REQUIRE(reported > 0, PA_GENERAL_ERROR, "the device reports no allocation granularity");
+        // address space for as much as the device could ever hold, shared between the tensors in proportion to their
+        // block sizes
+        size_t free_b = 0, total_b = 0;
+        HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        // A tensor's memory is mapped in pieces of one size, each at a multiple of that size: on this device pieces
+        // of differing sizes behind one another were refused now and then (hipMemSetAccess: invalid argument), and so
+        // were pieces at offsets aligned only to the 4 KiB the runtime reports; equal pieces never were.  The size is
+        // a power of two near 1/1024 of the tensor's address range, between 2 MiB and 64 MiB: at most about a
+        // thousand pieces per tensor (each costs about 60 us to create and map), at most one piece per tensor unused.
+        size_t piece = (size_t)2 << 20;
+        while (piece < ((size_t)64 << 20) && piece < total_b / n_tensors / 1024) piece *= 2;
+        PA_REQUIRE(piece % reported == 0, PA_GENERAL_ERROR, "unexpected allocation granularity");
+        c->granularity = piece;
+        const uint64_t all = c->all_block_bytes();
+        for (size_t t = 0; t < n_tensors; ++t) {
+            const size_t share = (size_t)((double)total_b * ((double)c->block_bytes[t] / (double)all));
+            c->reserved[t] = (share + piece - 1) / piece * piece;
+            HIP_CHECK(hipMemAddressReserve(&c->tensor(t), c->reserved[t], c->granularity, nullptr, 0));
+        }
+        // for the copy kernel: the base addresses, then the block sizes
+        std::vector<uint64_t> table(2 * n_tensors);
+        for (size_t t = 0; t < n_tensors; ++t) {
+            table[t] = (uint64_t)(uintptr_t)c->tensor(t);
+            table[n_tensors + t] = c->block_bytes[t];
+        }
+        c->base_table.reserve(table.size() * sizeof(uint64_t));
+        HIP_CHECK(hipMemcpy(c->base_table.p, table.data(), table.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    } catch (...) {
+        destroy_kv_cache(c);
+        throw;
+    }
+    *out = c;
+}
+}  // namespace
+
 int32_t pa_kv_cache_create(const pa_config* cfg, pa_kv_cache** out) {
     return guarded<NoObj>(nullptr, [&] {
         PA_REQUIRE(out, PA_INVALID_C_PARAM, "out is null");
         *out = nullptr;
         check_config(cfg);
-        HIP_CHECK(hipSetDevice(cfg->device));
-        pa_kv_cache* c = new pa_kv_cache();
-        c->cfg = *cfg;
-        const size_t n_tensors = 2 * (size_t)cfg->num_layers;
-        c->key.assign(cfg->num_layers, nullptr);
-        c->value.assign(cfg->num_layers, nullptr);
-        c->chunks.assign(n_tensors, {});
-        try {
-            PA_REQUIRE(c->layer_block_bytes() % 16 == 0, PA_NOT_IMPLEMENTED, "a block of one layer must be a multiple of 16 bytes");
-            const hipMemAllocationProp prop = device_memory_prop(cfg->device);
-            size_t reported = 0;
-            HIP_CHECK(hipMemGetAllocationGranularity(&reported, &prop, hipMemAllocationGranularityRecommended));
-            PA_REQUIRE(reported > 0, PA_GENERAL_ERROR, "the device reports no allocation granularity");
-            // address space for as much as the device could ever hold, shared evenly between the tensors
-            size_t free_b = 0, total_b = 0;
-            HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-            // A tensor's memory is mapped in pieces of one size, each at a multiple of that size: on this device pieces
-            // of differing sizes behind one another were refused now and then (hipMemSetAccess: invalid argument), and so
-            // were pieces at offsets aligned only to the 4 KiB the runtime reports; equal pieces never were.  The size is
-            // a power of two near 1/1024 of the tensor's address range, between 2 MiB and 64 MiB: at most about a
-            // thousand pieces per tensor (each costs about 60 us to create and map), at most one piece per tensor unused.
-            size_t piece = (size_t)2 << 20;
-            while (piece < ((size_t)64 << 20) && piece < total_b / n_tensors / 1024) piece *= 2;
-            PA_REQUIRE(piece % reported == 0, PA_GENERAL_ERROR, "unexpected allocation granularity");
-            c->granularity = piece;
-            c->reserved = (total_b / n_tensors + piece - 1) / piece * piece;
-            for (size_t t = 0; t < n_tensors; ++t)
-                HIP_CHECK(hipMemAddressReserve(&c->tensor(t), c->reserved, c->granularity, nullptr, 0));
-            std::vector<void*> bases(n_tensors);
-            for (size_t t = 0; t < n_tensors; ++t) bases[t] = c->tensor(t);
-            c->base_table.reserve(n_tensors * sizeof(void*));
-            HIP_CHECK(hipMemcpy(c->base_table.p, bases.data(), n_tensors * sizeof(void*), hipMemcpyHostToDevice));
-        } catch (...) {
-            destroy_kv_cache(c);
-            throw;
-        }
-        *out = c;
+        pa_kv_layer_desc one{};
+        one.key = pa_kv_tensor_desc{cfg->num_kv_heads, cfg->block_size, cfg->head_size, cfg->kv_cache_dtype};
+        one.value = pa_kv_tensor_desc{cfg->num_kv_heads, cfg->block_size, v_head(*cfg), v_dtype(*cfg)};
+        const std::vector<pa_kv_layer_desc> layers((size_t)cfg->num_layers, one);
+        create_kv_cache(cfg->device, cfg->stream, layers.data(), cfg->num_layers, out);
     });
+}
+
+int32_t pa_kv_cache_create_layers(int32_t device, void* stream, const pa_kv_layer_desc* layers, int32_t num_layers,
+                                  pa_kv_cache** out) {
+    return guarded<NoObj>(nullptr, [&] { create_kv_cache(device, stream, layers, num_layers, out); });
 }
 
 void pa_kv_cache_destroy(pa_kv_cache* c) {
@@ -1643,9 +1715,7 @@ void pa_kv_cache_destroy(pa_kv_cache* c) {
 
 const char* pa_kv_cache_last_error(const pa_kv_cache* c) { return c ? c->error.c_str() : g_last_error.c_str(); }
 
-uint64_t pa_kv_cache_block_bytes(const pa_kv_cache* c) {
-    return c ? 2ull * c->layer_block_bytes() * (uint64_t)c->cfg.num_layers : 0;
-}
+uint64_t pa_kv_cache_block_bytes(const pa_kv_cache* c) { return c ? c->all_block_bytes() : 0; }
 
 uint64_t pa_kv_cache_num_blocks(const pa_kv_cache* c) { return c ? c->num_blocks : 0; }
 
@@ -1656,13 +1726,17 @@ int32_t pa_kv_cache_allocate(pa_kv_cache* c, uint64_t num_kv_blocks) {
         HIP_CHECK(hipSetDevice(c->cfg.device));
         hipStream_t s = static_cast<hipStream_t>(c->cfg.stream);
         const char* too_large = "Requested KV-cache size is larger than available memory size on the system.";
-        const uint64_t bb = c->layer_block_bytes();
-        PA_REQUIRE(num_kv_blocks <= c->reserved / bb, PA_NOT_ALLOCATED, too_large);
-        const size_t need = ((size_t)(num_kv_blocks * bb) + c->granularity - 1) / c->granularity * c->granularity;
-        if (need > c->mapped) {
+        const size_t n_tensors = c->chunks.size(), piece = c->granularity;
+        // what every tensor needs mapped, and how many new pieces that is
+        std::vector<size_t> need(n_tensors), first_new(n_tensors + 1, 0);
+        for (size_t t = 0; t < n_tensors; ++t) {
+            PA_REQUIRE(num_kv_blocks <= c->reserved[t] / c->block_bytes[t], PA_NOT_ALLOCATED, too_large);
+            need[t] = ((size_t)(num_kv_blocks * c->block_bytes[t]) + piece - 1) / piece * piece;
+            first_new[t + 1] = first_new[t] + (need[t] > c->mapped[t] ? (need[t] - c->mapped[t]) / piece : 0);
+        }
+        const size_t n_fresh = first_new[n_tensors];
+        if (n_fresh > 0) {
             // memory for every tensor first, then the mappings: a failure anywhere leaves the cache as it was
-            const size_t add = need - c->mapped, n_tensors = c->chunks.size(), piece = c->granularity;
-            const size_t per_tensor = add / piece, n_fresh = per_tensor * n_tensors;
             const hipMemAllocationProp prop = device_memory_prop(c->cfg.device);
             std::vector<size_t> before(n_tensors);
             for (size_t t = 0; t < n_tensors; ++t) before[t] = c->chunks[t].size();
@@ -1683,28 +1757,31 @@ int32_t pa_kv_cache_allocate(pa_kv_cache* c, uint64_t num_kv_blocks) {
             hipMemAccessDesc access{};
             access.location = prop.location;
             access.flags = hipMemAccessFlagsProtReadWrite;
-            for (size_t i = 0; i < n_fresh; ++i) {
-                const size_t t = i / per_tensor, off = c->mapped + (i % per_tensor) * piece;
-                uint8_t* at = static_cast<uint8_t*>(c->tensor(t)) + off;
-                hipError_t e = hipMemMap(at, piece, 0, fresh[i], 0);
-                bool listed = false;
-                if (e == hipSuccess) {
-                    c->chunks[t].push_back({fresh[i], off, piece});
-                    listed = true;
-                    e = hipMemSetAccess(at, piece, &access, 1);
-                }
-                if (e != hipSuccess) {
-                    (void)hipGetLastError();
-                    for (size_t u = listed ? i + 1 : i; u < n_fresh; ++u) (void)hipMemRelease(fresh[u]);
-                    drop_chunks(c, before);
-                    throw StatusError(PA_NOT_ALLOCATED, std::string("mapping KV-cache memory failed: ") + hipGetErrorString(e));
+            for (size_t t = 0; t < n_tensors; ++t) {
+                for (size_t i = first_new[t]; i < first_new[t + 1]; ++i) {
+                    const size_t off = c->mapped[t] + (i - first_new[t]) * piece;
+                    uint8_t* at = static_cast<uint8_t*>(c->tensor(t)) + off;
+                    hipError_t e = hipMemMap(at, piece, 0, fresh[i], 0);
+                    bool listed = false;
+                    if (e == hipSuccess) {
+                        c->chunks[t].push_back({fresh[i], off, piece});
+                        listed = true;
+                        e = hipMemSetAccess(at, piece, &access, 1);
+                    }
+                    if (e != hipSuccess) {
+                        (void)hipGetLastError();
+                        for (size_t u = listed ? i + 1 : i; u < n_fresh; ++u) (void)hipMemRelease(fresh[u]);
+                        drop_chunks(c, before);
+                        throw StatusError(PA_NOT_ALLOCATED, std::string("mapping KV-cache memory failed: ") + hipGetErrorString(e));
+                    }
                 }
             }
             // new blocks start as zeros (rows no token has been written to are then harmless in any format)
             // (a failure here also unmaps and releases what this call made: the next growth maps the same offsets)
             hipError_t ze = hipSuccess;
             for (size_t t = 0; t < n_tensors && ze == hipSuccess; ++t)
-                ze = hipMemsetAsync(static_cast<uint8_t*>(c->tensor(t)) + c->mapped, 0, add, s);
+                if (need[t] > c->mapped[t])
+                    ze = hipMemsetAsync(static_cast<uint8_t*>(c->tensor(t)) + c->mapped[t], 0, need[t] - c->mapped[t], s);
             if (ze == hipSuccess) ze = hipStreamSynchronize(s);
             if (ze != hipSuccess) {
                 (void)hipGetLastError();
@@ -1712,7 +1789,7 @@ int32_t pa_kv_cache_allocate(pa_kv_cache* c, uint64_t num_kv_blocks) {
                 drop_chunks(c, before);
                 throw StatusError(PA_GENERAL_ERROR, std::string("clearing new KV-cache memory failed: ") + hipGetErrorString(ze));
             }
-            c->mapped = need;
+            for (size_t t = 0; t < n_tensors; ++t) c->mapped[t] = std::max(c->mapped[t], need[t]);
         }
         c->num_blocks = num_kv_blocks;
     });
@@ -1765,9 +1842,10 @@ int32_t pa_kv_cache_copy_blocks(pa_kv_cache* c, const int32_t* src, const int32_
         c->pairs.reserve(list.size() * sizeof(int32_t));
         HIP_CHECK(hipMemcpyAsync(c->pairs.p, list.data(), list.size() * sizeof(int32_t), hipMemcpyHostToDevice, s));
         for (size_t k = 0; k + 1 < cuts.size(); ++k)
-            HIP_CHECK(pa::launch_copy_blocks(s, c->base_table.as<void*>(), (int)c->chunks.size(),
+            HIP_CHECK(pa::launch_copy_blocks(s, c->base_table.as<void*>(),
+                                             c->base_table.as<uint64_t>() + c->chunks.size(), (int)c->chunks.size(),
                                              c->pairs.as<int32_t>() + 2 * cuts[k], cuts[k + 1] - cuts[k],
-                                             c->layer_block_bytes()));
+                                             *std::max_element(c->block_bytes.begin(), c->block_bytes.end())));
         HIP_CHECK(hipStreamSynchronize(s));  // `list` is pageable and leaves scope; the reference's copy is synchronous too
     });
 }

@@ -12,14 +12,25 @@ from .paged_attention import dtype_code, row_bytes
 
 
 class KVCacheManager:
-    def __init__(self, num_layers, num_kv_heads, head_size, block_size=32, kv_cache_dtype="u8", device=0):
+    def __init__(self, num_layers, num_kv_heads, head_size, block_size=32, kv_cache_dtype="u8", device=0, layers=None):
+        """``layers``: instead of one shape for all, per layer ``((kv heads, block size, head size, type) of the key
+        cache, the same of the value cache)`` -- what the reference reads off every ``key_cache.<L>`` / ``value_cache.<L>``
+        input (kv_cache_manager.hpp:74-92)."""
         cfg = L.pa_config()
         cfg.device, cfg.num_heads, cfg.num_kv_heads, cfg.head_size = device, num_kv_heads, num_kv_heads, head_size
         cfg.block_size, cfg.query_dtype, cfg.kv_cache_dtype, cfg.num_layers = block_size, L.PA_F16, dtype_code(kv_cache_dtype), num_layers
         self.cfg = cfg
         self.row_bytes = row_bytes(head_size, kv_cache_dtype)
         h = C.c_void_p()
-        L.check(L.lib().pa_kv_cache_create(C.byref(cfg), C.byref(h)), None)
+        if layers is None:
+            L.check(L.lib().pa_kv_cache_create(C.byref(cfg), C.byref(h)), None)
+        else:
+            assert len(layers) == num_layers
+            descs = (L.pa_kv_layer_desc * num_layers)()
+            for d, (k, v) in zip(descs, layers):
+                d.key = L.pa_kv_tensor_desc(k[0], k[1], k[2], dtype_code(k[3]))
+                d.value = L.pa_kv_tensor_desc(v[0], v[1], v[2], dtype_code(v[3]))
+            L.check(L.lib().pa_kv_cache_create_layers(device, None, descs, num_layers, C.byref(h)), None)
         self._h = h
 
     def __del__(self):

@@ -11,7 +11,7 @@ import numpy as np
 
 from . import _lib as L
 
-_DTYPES = {"f16": L.PA_F16, "bf16": L.PA_BF16, "u8": L.PA_U8}
+_DTYPES = {"f16": L.PA_F16, "bf16": L.PA_BF16, "u8": L.PA_U8, "u4": L.PA_U4}
 
 
 def dtype_code(name):
@@ -19,7 +19,9 @@ def dtype_code(name):
 
 
 def row_bytes(head_size, kv_cache_dtype):
-    return head_size + 8 if dtype_code(kv_cache_dtype) == L.PA_U8 else 2 * head_size
+    """Bytes of one cached row: 16-bit values, or `f32 scale | f32 zero-point` and the codes (u8: one byte each, u4: two per byte)."""
+    dt = dtype_code(kv_cache_dtype)
+    return head_size + 8 if dt == L.PA_U8 else head_size // 2 + 8 if dt == L.PA_U4 else 2 * head_size
 
 
 def _i32(a):
@@ -32,11 +34,15 @@ def _p32(a):
 
 class PagedAttention:
     def __init__(self, num_heads, num_kv_heads, head_size, block_size=32, query_dtype="f16", kv_cache_dtype="u8",
-                 num_layers=1, device=0, stream=None):
+                 num_layers=1, device=0, stream=None, v_head_size=None, value_cache_dtype=None):
+        """``v_head_size`` / ``value_cache_dtype``: head size and precision of ``value_cache.<L>`` where they differ
+        from the key side's (``head_size`` / ``kv_cache_dtype``)."""
         cfg = L.pa_config()
         cfg.device, cfg.num_heads, cfg.num_kv_heads, cfg.head_size = device, num_heads, num_kv_heads, head_size
         cfg.block_size, cfg.query_dtype, cfg.kv_cache_dtype = block_size, dtype_code(query_dtype), dtype_code(kv_cache_dtype)
         cfg.num_layers = num_layers
+        cfg.v_head_size = 0 if v_head_size is None else int(v_head_size)
+        cfg.value_cache_dtype_p1 = 0 if value_cache_dtype is None else 1 + dtype_code(value_cache_dtype)
         cfg.stream = C.c_void_p(int(getattr(stream, "cuda_stream", stream))) if stream is not None else None
         self.cfg = cfg
         h = C.c_void_p()

@@ -12,7 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libpa_oracle.so")
 
-DT_F16, DT_BF16, DT_U8 = 0, 1, 2
+DT_F16, DT_BF16, DT_U8, DT_U4 = 0, 1, 2, 3
 MODE_SUM, MODE_NORM_SUM, MODE_ADAPTIVE_RKV = 0, 1, 2
 
 
@@ -127,8 +127,15 @@ def quantize_row_u8(x):
     return row
 
 
+def quantize_row_u4(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    row = np.zeros(x.size // 2 + 8, dtype=np.uint8)
+    lib().orc_quantize_row_u4(_ptr(x, C.c_float), C.c_int32(x.size), _ptr(row, C.c_uint8))
+    return row
+
+
 def row_bytes(D, cache_dtype):
-    return D + 8 if cache_dtype == DT_U8 else 2 * D
+    return D + 8 if cache_dtype == DT_U8 else D // 2 + 8 if cache_dtype == DT_U4 else 2 * D
 
 
 def kv_append(key, value, src_dtype, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,
@@ -143,6 +150,42 @@ def kv_append(key, value, src_dtype, key_cache, value_cache, cache_dtype, past_l
         C.c_int32(B), C.c_int32(Hkv), C.c_int32(D), C.c_int32(bs))
     if rc != 0:
         raise RuntimeError(_err())
+
+
+def kv_append_kv(key, value, src_dtype, key_cache, value_cache, k_dtype, v_dtype, past_lens, subsequence_begins,
+                 block_indices, block_indices_begins, Hkv, Dk, Dv, bs):
+    """kv_append with a head size and an element type per tensor: key [T, Hkv*Dk], value [T, Hkv*Dv]."""
+    rc = lib().orc_kv_append_kv(
+        _ptr(key, C.c_uint16), _ptr(value, C.c_uint16), C.c_int32(src_dtype), _ptr(key_cache, C.c_uint8),
+        _ptr(value_cache, C.c_uint8), C.c_int32(k_dtype), C.c_int32(v_dtype), C.c_int64(key_cache.shape[0]),
+        _ptr(past_lens, C.c_int32), _ptr(subsequence_begins, C.c_int32), _ptr(block_indices, C.c_int32),
+        _ptr(block_indices_begins, C.c_int32), C.c_int32(len(past_lens)), C.c_int32(Hkv), C.c_int32(Dk), C.c_int32(Dv),
+        C.c_int32(bs))
+    if rc != 0:
+        raise RuntimeError(_err())
+
+
+def paged_attention_kv(query, q_dtype, key_cache, value_cache, k_dtype, v_dtype, past_lens, subsequence_begins,
+                       block_indices, block_indices_begins, Hq, Hkv, Dk, Dv, bs, scale, sliding_window=0,
+                       score_aggregation_window=None, want_scores=True, num_threads=1):
+    """paged_attention with a head size and an element type per tensor: query [T, Hq*Dk], out [T, Hq*Dv]."""
+    B = len(past_lens)
+    T = int(subsequence_begins[-1])
+    out = np.zeros((T, Hq * Dv), dtype=np.float32)
+    out16 = np.zeros((T, Hq * Dv), dtype=np.uint16)
+    total = int(np.sum(past_lens.astype(np.int64)) + T)
+    scores = np.zeros(total, dtype=np.float32) if want_scores else None
+    saw = None if score_aggregation_window is None else np.ascontiguousarray(score_aggregation_window, dtype=np.int32)
+    rc = lib().orc_paged_attention_kv(
+        _ptr(query, C.c_uint16), C.c_int32(q_dtype), _ptr(key_cache, C.c_uint8), _ptr(value_cache, C.c_uint8),
+        C.c_int32(k_dtype), C.c_int32(v_dtype), C.c_int64(key_cache.shape[0]), _ptr(past_lens, C.c_int32),
+        _ptr(subsequence_begins, C.c_int32), _ptr(block_indices, C.c_int32), _ptr(block_indices_begins, C.c_int32),
+        _ptr(saw, C.c_int32), C.c_int32(B), C.c_int32(Hq), C.c_int32(Hkv), C.c_int32(Dk), C.c_int32(Dv), C.c_int32(bs),
+        C.c_float(scale), C.c_int32(sliding_window), _ptr(out, C.c_float), _ptr(out16, C.c_uint16),
+        _ptr(scores, C.c_float), C.c_int32(num_threads))
+    if rc != 0:
+        raise RuntimeError(_err())
+    return out, out16, scores
 
 
 def paged_attention(query, q_dtype, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,

@@ -34,6 +34,8 @@
 // behaviour is restated here; those functions are marked PARITY UNPINNED because
 // nothing the reference holds can pin them:
 //   orc_quantize_row_u8      PARITY UNPINNED vs the plugin (pinned by closed-form invariants only)
+//   orc_quantize_row_u4      PARITY UNPINNED vs the plugin (the same recipe with 15 levels, two codes per byte, high
+//                            nibble first; pinned by the same closed-form invariants)
 //   orc_kv_append            PARITY UNPINNED vs the plugin (pinned by brute-force gather/scatter)
 //   orc_paged_attention      PARITY UNPINNED vs the plugin (pinned against textbook SDPA in float64)
 //   orc_rotate_cache         PARITY UNPINNED vs the plugin (the re-rotation of cached K rows happens inside the op;
@@ -72,7 +74,7 @@
 
 namespace {
 
-enum { DT_F16 = 0, DT_BF16 = 1, DT_U8 = 2 };
+enum { DT_F16 = 0, DT_BF16 = 1, DT_U8 = 2, DT_U4 = 3 };
 
 // ---------------------------------------------------------------- 16-bit floats
 float half_to_float(uint16_t h) {
@@ -167,7 +169,37 @@ void quantize_row(const float* x, int D, uint8_t* row) {
     }
 }
 
-inline size_t row_bytes(int D, int dt) { return dt == DT_U8 ? (size_t)D + 8 : (size_t)D * 2; }
+// Row layout for a u4 cache, by token, per head: f32 scale | f32 zero-point | D / 2 bytes, element 2 i in the high
+// nibble of byte i and element 2 i + 1 in the low one.  Recipe as for u8 rows with 15 levels: scale = (max - min) / 15
+// (a zero range takes 1e-4), zp = -min / scale, code = clamp(rne(x * (1 / scale) + zp), 0, 15).
+// [Restated from memory of the OpenVINO CPU plugin's 4-bit KV quantisation, which is not in the reference tree:
+// PARITY UNPINNED, nibble order and rounding included.]
+void quantize_row_u4(const float* x, int D, uint8_t* row) {
+    float mn = x[0], mx = x[0];
+    for (int d = 1; d < D; ++d) {
+        mn = std::fmin(mn, x[d]);
+        mx = std::fmax(mx, x[d]);
+    }
+    float scale = (mx - mn) / 15.0f;
+    if (scale == 0.0f) scale = 0.0001f;
+    float zp = -mn / scale;
+    float inv = 1.0f / scale;
+    std::memcpy(row, &scale, 4);
+    std::memcpy(row + 4, &zp, 4);
+    for (int d = 0; d < D; d += 2) {
+        uint8_t c[2];
+        for (int e = 0; e < 2; ++e) {
+            float v = std::nearbyintf(std::fmaf(x[d + e], inv, zp));
+            v = std::fmin(std::fmax(v, 0.0f), 15.0f);
+            c[e] = (uint8_t)(int)v;
+        }
+        row[8 + d / 2] = (uint8_t)((c[0] << 4) | c[1]);
+    }
+}
+
+inline size_t row_bytes(int D, int dt) {
+    return dt == DT_U8 ? (size_t)D + 8 : dt == DT_U4 ? (size_t)D / 2 + 8 : (size_t)D * 2;
+}
 
 // Reads one cached row (block, head, slot) into f32.
 inline void load_cache_row(const uint8_t* cache, int dt, int64_t phys, int h, int slot, int Hkv, int bs, int D,
@@ -179,6 +211,14 @@ inline void load_cache_row(const uint8_t* cache, int dt, int64_t phys, int h, in
         std::memcpy(&scale, row, 4);
         std::memcpy(&zp, row + 4, 4);
         for (int d = 0; d < D; ++d) dst[d] = ((float)row[8 + d] - zp) * scale;
+    } else if (dt == DT_U4) {
+        float scale, zp;
+        std::memcpy(&scale, row, 4);
+        std::memcpy(&zp, row + 4, 4);
+        for (int d = 0; d < D; ++d) {
+            const uint8_t byte = row[8 + d / 2];
+            dst[d] = ((float)((d & 1) ? (byte & 15) : (byte >> 4)) - zp) * scale;
+        }
     } else {
         const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
         for (int d = 0; d < D; ++d) dst[d] = load16(r16 + d, dt);
@@ -665,13 +705,27 @@ void orc_quantize_row_u8(const float* x, int32_t D, uint8_t* row) {
 //   caches:    [num_blocks, Hkv, block, row] with row = D*2 bytes (16-bit cache) or D+8 bytes (u8)
 // Token t of sequence b lands in slot past_lens[b] + t: physical block
 // block_indices[block_indices_begins[b] + slot / block], offset slot % block.
-int32_t orc_kv_append(const uint16_t* key, const uint16_t* value, int32_t src_dtype, uint8_t* key_cache,
-                      uint8_t* value_cache, int32_t cache_dtype, int64_t num_blocks, const int32_t* past_lens,
-                      const int32_t* subsequence_begins, const int32_t* block_indices,
-                      const int32_t* block_indices_begins, int32_t B, int32_t Hkv, int32_t D, int32_t bs) {
+static void append_row(const uint16_t* src, int src_dtype, uint8_t* dst, int cache_dtype, int D, std::vector<float>& tmp) {
+    if (cache_dtype == DT_U8 || cache_dtype == DT_U4) {
+        for (int d = 0; d < D; ++d) tmp[d] = load16(src + d, src_dtype);
+        if (cache_dtype == DT_U8) quantize_row(tmp.data(), D, dst);
+        else quantize_row_u4(tmp.data(), D, dst);
+    } else if (cache_dtype == src_dtype) {
+        std::memcpy(dst, src, row_bytes(D, cache_dtype));
+    } else {
+        uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+        for (int d = 0; d < D; ++d) d16[d] = store16(load16(src + d, src_dtype), cache_dtype);
+    }
+}
+
+// The same with a head size and an element type per tensor: key [T, Hkv*Dk], value [T, Hkv*Dv]; key_cache rows of
+// Dk elements in k_dtype, value_cache rows of Dv elements in v_dtype (DT_U4 included).
+int32_t orc_kv_append_kv(const uint16_t* key, const uint16_t* value, int32_t src_dtype, uint8_t* key_cache,
+                         uint8_t* value_cache, int32_t k_dtype, int32_t v_dtype, int64_t num_blocks,
+                         const int32_t* past_lens, const int32_t* subsequence_begins, const int32_t* block_indices,
+                         const int32_t* block_indices_begins, int32_t B, int32_t Hkv, int32_t Dk, int32_t Dv, int32_t bs) {
     std::fesetround(FE_TONEAREST);
-    size_t rb = row_bytes(D, cache_dtype);
-    std::vector<float> tmp(D);
+    std::vector<float> tmp(std::max(Dk, Dv));
     for (int b = 0; b < B; ++b) {
         int q_len = subsequence_begins[b + 1] - subsequence_begins[b];
         int nblk = block_indices_begins[b + 1] - block_indices_begins[b];
@@ -682,23 +736,27 @@ int32_t orc_kv_append(const uint16_t* key, const uint16_t* value, int32_t src_dt
             if (phys < 0 || phys >= num_blocks) { g_error = "kv_append: physical block id out of range"; return -6; }
             size_t tok = (size_t)subsequence_begins[b] + t;
             for (int h = 0; h < Hkv; ++h) {
-                for (int which = 0; which < 2; ++which) {
-                    const uint16_t* src = (which ? value : key) + (tok * Hkv + h) * D;
-                    uint8_t* dst = (which ? value_cache : key_cache) + (((size_t)phys * Hkv + h) * bs + slot % bs) * rb;
-                    if (cache_dtype == DT_U8) {
-                        for (int d = 0; d < D; ++d) tmp[d] = load16(src + d, src_dtype);
-                        quantize_row(tmp.data(), D, dst);
-                    } else if (cache_dtype == src_dtype) {
-                        std::memcpy(dst, src, rb);
-                    } else {
-                        uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
-                        for (int d = 0; d < D; ++d) d16[d] = store16(load16(src + d, src_dtype), cache_dtype);
-                    }
-                }
+                append_row(key + (tok * Hkv + h) * Dk, src_dtype,
+                           key_cache + (((size_t)phys * Hkv + h) * bs + slot % bs) * row_bytes(Dk, k_dtype), k_dtype, Dk, tmp);
+                append_row(value + (tok * Hkv + h) * Dv, src_dtype,
+                           value_cache + (((size_t)phys * Hkv + h) * bs + slot % bs) * row_bytes(Dv, v_dtype), v_dtype, Dv, tmp);
             }
         }
     }
     return 0;
+}
+
+int32_t orc_kv_append(const uint16_t* key, const uint16_t* value, int32_t src_dtype, uint8_t* key_cache,
+                      uint8_t* value_cache, int32_t cache_dtype, int64_t num_blocks, const int32_t* past_lens,
+                      const int32_t* subsequence_begins, const int32_t* block_indices,
+                      const int32_t* block_indices_begins, int32_t B, int32_t Hkv, int32_t D, int32_t bs) {
+    return orc_kv_append_kv(key, value, src_dtype, key_cache, value_cache, cache_dtype, cache_dtype, num_blocks, past_lens,
+                            subsequence_begins, block_indices, block_indices_begins, B, Hkv, D, D, bs);
+}
+
+void orc_quantize_row_u4(const float* x, int32_t D, uint8_t* row) {
+    std::fesetround(FE_TONEAREST);
+    quantize_row_u4(x, D, row);
 }
 
 // ------------------------------------------------------------------ attention
@@ -712,13 +770,17 @@ int32_t orc_kv_append(const uint16_t* key, const uint16_t* value, int32_t src_dt
 // With `retained` (sparse prefill, see orc_xattention_* below): retained[b] is null (dense) or, for the sequence's
 // query blocks I = past_b / xb .. (past_b + new_b - 1) / xb and key blocks J = 0 .. last I, bytes [Hq][nqb][nkb]; the
 // row at position p of head h then only sees positions j with retained[b][h][p / xb - past_b / xb][j / xb] != 0.
+// Head size and element type per tensor: query and key rows have D elements, value and output rows Dv; K rows are
+// read as cache_dtype, V rows as v_dtype.
 static int32_t paged_attention_impl(const uint16_t* query, int32_t q_dtype, const uint8_t* key_cache,
                             const uint8_t* value_cache, int32_t cache_dtype, int64_t num_blocks,
                             const int32_t* past_lens, const int32_t* subsequence_begins, const int32_t* block_indices,
                             const int32_t* block_indices_begins, const int32_t* score_aggregation_window, int32_t B,
                             int32_t Hq, int32_t Hkv, int32_t D, int32_t bs, float scale, int32_t sliding_window,
                             float* out_f32, uint16_t* out16, float* scores, int32_t num_threads,
-                            const uint8_t* const* retained, int32_t xb) {
+                            const uint8_t* const* retained, int32_t xb, int32_t Dv = -1, int32_t v_dtype = -1) {
+    if (Dv < 0) Dv = D;
+    if (v_dtype < 0) v_dtype = cache_dtype;
     if (Hq % Hkv) { g_error = "Hq must be a multiple of Hkv"; return -14; }
     const int G = Hq / Hkv;
     std::vector<int64_t> score_off(B + 1, 0);
@@ -748,17 +810,17 @@ static int32_t paged_attention_impl(const uint16_t* query, int32_t q_dtype, cons
             const int32_t* table = block_indices + block_indices_begins[b];
             const int W = score_aggregation_window ? score_aggregation_window[b] : 1;
             // gather this head's K and V rows once, dequantised to f32
-            std::vector<float> K((size_t)kv_len * D), V((size_t)kv_len * D);
+            std::vector<float> K((size_t)kv_len * D), V((size_t)kv_len * Dv);
             for (int j = 0; j < kv_len; ++j) {
                 load_cache_row(key_cache, cache_dtype, table[j / bs], h, j % bs, Hkv, bs, D, &K[(size_t)j * D]);
-                load_cache_row(value_cache, cache_dtype, table[j / bs], h, j % bs, Hkv, bs, D, &V[(size_t)j * D]);
+                load_cache_row(value_cache, v_dtype, table[j / bs], h, j % bs, Hkv, bs, Dv, &V[(size_t)j * Dv]);
             }
             std::vector<double>* sp = nullptr;
             if (scores) {
                 sp = &score_part[(size_t)b * Hkv + h];
                 sp->assign(kv_len, 0.0);
             }
-            std::vector<float> q(D), p(kv_len), acc(D);
+            std::vector<float> q(D), p(kv_len), acc(Dv);
             for (int i = 0; i < q_len; ++i) {
                 const int last = past + i;  // last visible position
                 const int first = (sliding_window > 0) ? std::max(0, last + 1 - sliding_window) : 0;
@@ -792,15 +854,15 @@ static int32_t paged_attention_impl(const uint16_t* query, int32_t q_dtype, cons
                     std::fill(acc.begin(), acc.end(), 0.0f);
                     for (int j = first; j <= last; ++j) {
                         const float w = p[j] * inv_l;
-                        const float* vr = &V[(size_t)j * D];
+                        const float* vr = &V[(size_t)j * Dv];
 #pragma omp simd
-                        for (int d = 0; d < D; ++d) acc[d] += w * vr[d];
+                        for (int d = 0; d < Dv; ++d) acc[d] += w * vr[d];
                         if (sp && i >= q_len - W) (*sp)[j] += (double)w;
                     }
-                    size_t o = ((size_t)(q0 + i) * Hq + hq) * D;
-                    if (out_f32) std::memcpy(out_f32 + o, acc.data(), sizeof(float) * D);
+                    size_t o = ((size_t)(q0 + i) * Hq + hq) * Dv;
+                    if (out_f32) std::memcpy(out_f32 + o, acc.data(), sizeof(float) * Dv);
                     if (out16)
-                        for (int d = 0; d < D; ++d) out16[o + d] = store16(acc[d], q_dtype);
+                        for (int d = 0; d < Dv; ++d) out16[o + d] = store16(acc[d], q_dtype);
                 }
             }
         }
@@ -827,6 +889,20 @@ int32_t orc_paged_attention(const uint16_t* query, int32_t q_dtype, const uint8_
     return paged_attention_impl(query, q_dtype, key_cache, value_cache, cache_dtype, num_blocks, past_lens,
                                 subsequence_begins, block_indices, block_indices_begins, score_aggregation_window, B, Hq,
                                 Hkv, D, bs, scale, sliding_window, out_f32, out16, scores, num_threads, nullptr, 0);
+}
+
+// ... with a head size and an element type per tensor (query / key rows of Dk elements, value / output rows of Dv)
+int32_t orc_paged_attention_kv(const uint16_t* query, int32_t q_dtype, const uint8_t* key_cache,
+                               const uint8_t* value_cache, int32_t k_dtype, int32_t v_dtype, int64_t num_blocks,
+                               const int32_t* past_lens, const int32_t* subsequence_begins, const int32_t* block_indices,
+                               const int32_t* block_indices_begins, const int32_t* score_aggregation_window, int32_t B,
+                               int32_t Hq, int32_t Hkv, int32_t Dk, int32_t Dv, int32_t bs, float scale,
+                               int32_t sliding_window, float* out_f32, uint16_t* out16, float* scores,
+                               int32_t num_threads) {
+    return paged_attention_impl(query, q_dtype, key_cache, value_cache, k_dtype, num_blocks, past_lens,
+                                subsequence_begins, block_indices, block_indices_begins, score_aggregation_window, B, Hq,
+                                Hkv, Dk, bs, scale, sliding_window, out_f32, out16, scores, num_threads, nullptr, 0, Dv,
+                                v_dtype);
 }
 
 // ------------------------------------------------------------------ XAttention (sparse prefill, importance estimate)

@@ -27,13 +27,13 @@ def frac_to_f32(fr):
     return np.float32(sign * float(Fraction(n) * Fraction(2) ** (e - 23)))
 
 
-def quantize_row_exact(x):
-    """u8 row of ``x`` (float32 values) by exact rational arithmetic: scale, zp, codes."""
+def quantize_row_exact(x, levels=255):
+    """u8 (``levels`` 255) or u4 (15) row of ``x`` (float32 values) by exact rational arithmetic: scale, zp, codes."""
     x = [np.float32(v) for v in x]
     mn, mx = min(x), max(x)
     # (mx - mn) is itself rounded to float32 before the division
     diff = frac_to_f32(Fraction(float(mx)) - Fraction(float(mn)))
-    scale = frac_to_f32(Fraction(float(diff)) / 255)
+    scale = frac_to_f32(Fraction(float(diff)) / levels)
     if scale == 0:
         scale = np.float32(0.0001)
     zp = frac_to_f32(-Fraction(float(mn)) / Fraction(float(scale)))
@@ -46,7 +46,7 @@ def quantize_row_exact(x):
         d = t - r
         if d > 0.5 or (d == 0.5 and int(r) % 2 == 1):
             r += 1
-        codes.append(int(min(max(r, 0), 255)))
+        codes.append(int(min(max(r, 0), levels)))
     return scale, zp, codes
 
 
@@ -62,17 +62,26 @@ def dequant_rows_u8(rows):
     return (rows[:, 8:].astype(np.float32) - zp) * scale
 
 
+def dequant_rows_u4(rows):
+    """rows uint8 [n, D/2+8] -> float32 [n, D]: element 2 i from the high nibble of byte i, 2 i + 1 from the low one."""
+    hdr = rows[:, :8].copy().view(np.float32)
+    scale, zp = hdr[:, 0:1], hdr[:, 1:2]
+    codes = np.stack([rows[:, 8:] >> 4, rows[:, 8:] & 15], axis=2).reshape(rows.shape[0], -1)
+    return (codes.astype(np.float32) - zp) * scale
+
+
 def attention_f64(q, K, V, past, scale, sliding_window, W):
     """Textbook attention in float64 for one sequence and one kv head.
 
-    q [q_len, G, D], K/V [kv_len, D] -> out [q_len, G, D], scores [kv_len] (sum over G heads and last W rows).
+    q [q_len, G, D], K [kv_len, D], V [kv_len, Dv] -> out [q_len, G, Dv], scores [kv_len] (sum over G heads and
+    last W rows).
     """
     q = q.astype(np.float64)
     K = K.astype(np.float64)
     V = V.astype(np.float64)
     q_len, G, D = q.shape
     kv_len = K.shape[0]
-    out = np.zeros((q_len, G, D))
+    out = np.zeros((q_len, G, V.shape[1]))
     scores = np.zeros(kv_len)
     for i in range(q_len):
         last = past + i

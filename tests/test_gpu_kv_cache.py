@@ -249,3 +249,38 @@ def test_copy_blocks_of_a_whole_batch_is_exact_and_ordered(env):
     got = _read(hip, mgr.get_key_cache(5), nb * per_layer).reshape(nb, per_layer)
     for blk in (1, 2, 590, 591):
         assert np.array_equal(got[blk], base0[0]), blk
+
+
+def test_shape_and_precision_per_layer_and_per_tensor(env):
+    """Layers whose K and V tensors differ in kv heads, head size and precision (u4 included): block bytes add up as
+    the reference adds them (kv_cache_manager.hpp:74-92), growth keeps every tensor's blocks, copy_blocks copies each
+    tensor's own block size."""
+    pkg, _, hip = env
+    layers = [((8, 32, 128, "u8"), (8, 32, 128, "u8")), ((4, 32, 192, "bf16"), (4, 32, 128, "u4")),
+              ((2, 32, 80, "f16"), (2, 32, 256, "u8")), ((8, 32, 64, "u4"), (8, 32, 64, "f16"))]
+    rb = {"u8": lambda d: d + 8, "u4": lambda d: d // 2 + 8, "f16": lambda d: 2 * d, "bf16": lambda d: 2 * d}
+    per = [[h * b * rb[t](d) for (h, b, d, t) in kv] for kv in layers]
+    mgr = pkg.KVCacheManager(len(layers), 8, 128, 32, "u8", layers=layers)
+    assert mgr.get_block_size_in_bytes() == sum(sum(p) for p in per)
+    nb = 40
+    mgr.allocate_cache_if_needed(nb)
+    rng = np.random.default_rng(11)
+    content = {}
+    for l in range(len(layers)):
+        for w in range(2):
+            content[l, w] = rng.integers(0, 256, (nb, per[l][w]), dtype=np.uint8)
+            _write(hip, (mgr.get_key_cache(l), mgr.get_value_cache(l))[w], content[l, w])
+    ptrs = [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(len(layers))]
+    mgr.allocate_cache_if_needed(4 * nb)  # growth: same addresses, old blocks kept, new ones zero
+    assert ptrs == [(mgr.get_key_cache(l), mgr.get_value_cache(l)) for l in range(len(layers))]
+    mgr.copy_blocks({3: [nb + 5, 7], 9: [4 * nb - 1]})
+    for l in range(len(layers)):
+        for w in range(2):
+            got = _read(hip, ptrs[l][w], 4 * nb * per[l][w]).reshape(4 * nb, per[l][w])
+            want = np.zeros_like(got)
+            want[:nb] = content[l, w]
+            want[nb + 5] = want[7] = content[l, w][3]
+            want[4 * nb - 1] = content[l, w][9]
+            assert np.array_equal(got, want), (l, w)
+    with pytest.raises(pkg.PaError):
+        pkg.KVCacheManager(1, 8, 128, 32, "u8", layers=[((8, 32, 0, "u8"), (8, 32, 128, "u8"))])

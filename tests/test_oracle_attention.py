@@ -104,6 +104,123 @@ def test_quantize_row_invariants():
 
 
 # ------------------------------------------------------------------------------------------- append = scatter
+# ------------------------------------------------------------------------------------------- u4 rows
+@pytest.mark.parametrize("seed", range(5))
+def test_quantize_row_u4_matches_exact_rational(seed):
+    rng = np.random.default_rng(300 + seed)
+    D = [8, 16, 80, 128, 256][seed]
+    x = rng.standard_normal(D).astype(np.float16).astype(np.float32)
+    if seed == 3:
+        x[rng.integers(0, D, 3)] = np.float32([8.0, -8.0, 8.0])
+    row = O.quantize_row_u4(x)
+    assert row.size == D // 2 + 8
+    scale, zp, codes = R.quantize_row_exact(x, levels=15)
+    assert row[:4].view(np.float32)[0] == scale
+    assert row[4:8].view(np.float32)[0] == zp
+    got = np.stack([row[8:] >> 4, row[8:] & 15], axis=1).reshape(-1)  # element 2 i in the high nibble of byte i
+    assert list(got) == codes
+
+
+def test_quantize_row_u4_invariants():
+    rng = np.random.default_rng(8)
+    for D in (8, 64, 96, 128):
+        x = (rng.standard_normal(D) * 3).astype(np.float32)
+        row = O.quantize_row_u4(x)
+        sc, zp = row[:8].view(np.float32)
+        codes = np.stack([row[8:] >> 4, row[8:] & 15], axis=1).reshape(-1)
+        assert codes.min() == 0 and codes.max() == 15  # the extremes land on the ends of the range
+        assert np.argmin(x) in np.flatnonzero(codes == 0) and np.argmax(x) in np.flatnonzero(codes == 15)
+        deq = (codes.astype(np.float32) - zp) * sc
+        assert np.all(np.abs(deq - x) <= 0.5 * sc * 1.001 + 1e-6)  # half a quantisation step
+        assert np.array_equal(R.dequant_rows_u4(row[None])[0], deq)
+    const = O.quantize_row_u4(np.full(16, 2.5, np.float32))  # a zero range takes the fixed scale
+    assert const[:4].view(np.float32)[0] == np.float32(0.0001)
+    # exact ties round to even: min 0, max 15 -> scale 1, zp 0
+    x = np.array([0.0, 15.0, 0.5, 1.5, 2.5, 3.5, 13.5, 14.5], np.float32)
+    row = O.quantize_row_u4(x)
+    assert list(np.stack([row[8:] >> 4, row[8:] & 15], axis=1).reshape(-1)) == [0, 15, 0, 2, 2, 4, 14, 14]
+
+
+KV_MIXES = [
+    # (Dk, Dv, key cache type, value cache type): head sizes and precisions that differ between the two tensors
+    (80, 80, "f16", "f16"), (96, 96, "u8", "u8"), (256, 256, "bf16", "bf16"), (128, 64, "u8", "f16"),
+    (64, 128, "f16", "u8"), (192, 128, "bf16", "u4"), (128, 128, "u4", "u4"), (72, 40, "u4", "bf16"),
+]
+
+
+@pytest.mark.parametrize("Dk,Dv,kd,vd", KV_MIXES)
+def test_attention_with_a_head_size_and_type_per_tensor_matches_float64(Dk, Dv, kd, vd):
+    """The per-tensor form of the checker (key rows of Dk elements in one type, value rows of Dv in another) against
+    the float64 textbook form over rows dequantised independently here; the append is checked row by row."""
+    dts = {"f16": O.DT_F16, "bf16": O.DT_BF16, "u8": O.DT_U8, "u4": O.DT_U4}
+    kdt, vdt = dts[kd], dts[vd]
+    qdt = O.DT_BF16 if "bf16" in (kd, vd) else O.DT_F16
+    rng = np.random.default_rng(Dk * 7 + Dv)
+    B, Hq, Hkv, bs = 3, 6, 2, 16
+    G = Hq // Hkv
+    past = np.array([0, 37, 90], np.int32)
+    new = np.array([21, 1, 5], np.int32)
+    sb = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    nblk = (past + new + bs - 1) // bs
+    bib = np.concatenate([[0], np.cumsum(nblk)]).astype(np.int32)
+    pool = 2 * int(bib[-1]) + 1
+    table = rng.permutation(pool)[:bib[-1]].astype(np.int32)
+    kc = np.zeros((pool, Hkv, bs, O.row_bytes(Dk, kdt)), np.uint8)
+    vc = np.zeros((pool, Hkv, bs, O.row_bytes(Dv, vdt)), np.uint8)
+    tot = past + new
+    asb = np.concatenate([[0], np.cumsum(tot)]).astype(np.int32)
+    k_all = rng.standard_normal((int(asb[-1]), Hkv, Dk)).astype(np.float32)
+    v_all = rng.standard_normal((int(asb[-1]), Hkv, Dv)).astype(np.float32)
+    kb, vb = O.to_bits(k_all.reshape(-1, Hkv * Dk), qdt), O.to_bits(v_all.reshape(-1, Hkv * Dv), qdt)
+    O.kv_append_kv(kb, vb, qdt, kc, vc, kdt, vdt, np.zeros(B, np.int32), asb, table, bib, Hkv, Dk, Dv, bs)
+
+    def rows(cache, D, dt, b, h):
+        r = R.gather_rows(cache, table[bib[b]:bib[b + 1]], int(tot[b]), h, bs)
+        if dt == O.DT_U8:
+            return R.dequant_rows_u8(r)
+        if dt == O.DT_U4:
+            return R.dequant_rows_u4(r)
+        return O.from_bits(r.reshape(int(tot[b]), -1).view(np.uint16), dt)
+
+    # the append: every row is what its type's recipe makes of the source row
+    src_k = O.from_bits(kb, qdt).reshape(-1, Hkv, Dk)
+    src_v = O.from_bits(vb, qdt).reshape(-1, Hkv, Dv)
+    for b in range(B):
+        for h in range(Hkv):
+            for cache, D, dt, src in ((kc, Dk, kdt, src_k), (vc, Dv, vdt, src_v)):
+                got = R.gather_rows(cache, table[bib[b]:bib[b + 1]], int(tot[b]), h, bs)
+                for j in (0, int(tot[b]) - 1):
+                    x = src[asb[b] + j, h]
+                    if dt == O.DT_U8:
+                        assert np.array_equal(got[j], O.quantize_row_u8(x))
+                    elif dt == O.DT_U4:
+                        assert np.array_equal(got[j], O.quantize_row_u4(x))
+                    else:
+                        assert np.array_equal(got[j].view(np.uint16), O.to_bits(x[None], dt)[0])
+    q = O.to_bits(rng.standard_normal((int(sb[-1]), Hq * Dk)).astype(np.float32), qdt)
+    scale = float(1.0 / np.sqrt(Dk))
+    W = np.array([3, 1, 2], np.int32)
+    out, out16, scores = O.paged_attention_kv(q, qdt, kc, vc, kdt, vdt, past, sb, table, bib, Hq, Hkv, Dk, Dv, bs, scale,
+                                              0, W, True, 4)
+    assert out.shape == (int(sb[-1]), Hq * Dv)
+    qf = O.from_bits(q, qdt).reshape(-1, Hq, Dk)
+    so = np.concatenate([[0], np.cumsum(tot)])
+    for b in range(B):
+        sc_ref = np.zeros(int(tot[b]))
+        for h in range(Hkv):
+            o, s = R.attention_f64(qf[sb[b]:sb[b + 1], h * G:(h + 1) * G], rows(kc, Dk, kdt, b, h), rows(vc, Dv, vdt, b, h),
+                                   int(past[b]), scale, 0, int(W[b]))
+            got = out[sb[b]:sb[b + 1]].reshape(-1, Hq, Dv)[:, h * G:(h + 1) * G]
+            np.testing.assert_allclose(got, o, rtol=2e-5, atol=2e-5)
+            sc_ref += s
+        np.testing.assert_allclose(scores[so[b]:so[b + 1]], sc_ref, rtol=2e-5, atol=2e-5)
+    # ... and equal head sizes and types give the bits of the plain form
+    if Dk == Dv and kdt == vdt and kdt != O.DT_U4:
+        out2, out16_2, scores2 = O.paged_attention(q, qdt, kc, vc, kdt, past, sb, table, bib, Hq, Hkv, Dk, bs, scale, 0, W,
+                                                   True, 4)
+        assert np.array_equal(out16, out16_2) and np.array_equal(scores, scores2)
+
+
 @pytest.mark.parametrize("cache_dtype,src_dtype", [(O.DT_U8, O.DT_F16), (O.DT_F16, O.DT_F16), (O.DT_BF16, O.DT_BF16),
                                                    (O.DT_U8, O.DT_BF16)])
 def test_kv_append_is_a_paged_scatter(cache_dtype, src_dtype):

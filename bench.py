@@ -54,6 +54,8 @@ def parse():
     ap.add_argument("--layers", type=int, default=32,
                     help="decoder layers of the eviction leg of --config 4 (score registration and eviction run over "
                          "every layer of every sequence in one call)")
+    ap.add_argument("--evict-modes", default="norm_sum,kvcrush,adaptive_rkv",
+                    help="eviction legs of --config 4 beside NORM_SUM: kvcrush, adaptive_rkv (comma separated)")
     ap.add_argument("--diversity", type=int, default=0, metavar="TOKENS",
                     help="adds a leg: ADAPTIVE_RKV block diversity over an evictable area of this many tokens (a "
                          "multiple of 32) of every sequence, behind a start area of 32 tokens")
@@ -150,31 +152,63 @@ def cpu_model():
         got.get("stepping", "?"), got.get("cpu MHz", "?"))
 
 
-def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, layers):
+def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, layers, mode="norm_sum"):
     """Score accumulation + eviction on the device for the scoring workload, every layer of every sequence in one
     call (the layers share one scores tensor here): the first registration sees the whole 8193-token context and
-    evicts down to max_cache_size; the steady state registers a 1024-token cache's scores and evicts one block.
+    evicts down to max_cache_size; the steady state registers a 1024-token cache's scores plus one block of new
+    tokens and evicts one block per sequence and layer in every timed step (the step that comes up once per
+    block_size generated tokens; the steps between register only).
     Times are host wall clock around the C-ABI calls (upload of the per-pair entries, launches, read-back of the
-    evicted block lists included), buffers preallocated."""
+    evicted block lists included), buffers preallocated.
+    mode: "norm_sum"; "kvcrush" (NORM_SUM with a KVCrush budget of 8 blocks, MEAN anchor: some of the chosen blocks
+    stay as representatives); "adaptive_rkv" (a block diversity matrix is registered before every eviction, as the
+    pipeline does with the op's `adaptive_rkv_diversity.<L>` output -- synthetic values here, one tensor for all
+    layers; its first eviction runs over 2 layers, the diversity of 8000 evictable tokens being 8 MB per pair)."""
     import ctypes as C
     from openvino_genai_amd import _lib as L
     B, bs = spec["B"], spec["bs"]
-    cfg = pkg.CacheEvictionConfig(32, 128, 1024, pkg.AggregationMode.NORM_SUM, False, 0)
-    ev = pkg.Evictor(cfg, bs, layers, 7, max_sequences=B, max_tracked_tokens=8448, device=0,
-                     stream=torch.cuda.current_stream(dev))
+    rkv = mode == "adaptive_rkv"
+    agg = pkg.AggregationMode.ADAPTIVE_RKV if rkv else pkg.AggregationMode.NORM_SUM
+    crush = pkg.KVCrushConfig(8, pkg.KVCrushAnchorPointMode.MEAN) if mode == "kvcrush" else None
+    cfg = pkg.CacheEvictionConfig(32, 128, 1024, agg, False, 0, crush)
+    cfg_every = pkg.CacheEvictionConfig(32, 128, 1024, agg, False, 0, pkg.KVCrushConfig(1, pkg.KVCrushAnchorPointMode.MEAN))
     lib = L.lib()
     slots = np.arange(B, dtype=np.int32)
-    ptrs = (C.c_void_p * layers)(*[C.c_void_p(scores.data_ptr())] * layers)
-    counts = np.zeros(B * layers, np.int32)
-    blocks = np.zeros(B * layers * 256, np.int32)
     p32 = lambda a: a.ctypes.data_as(C.POINTER(C.c_int32))
+    p64 = lambda a: a.ctypes.data_as(C.POINTER(C.c_int64))
+    start = 32
 
-    def register(offsets):
-        L.check(lib.pa_evictor_register_scores(ev._h, B, p32(slots), ptrs, offsets.ctypes.data_as(C.POINTER(C.c_int64)), None),
-                lib.pa_evictor_last_error, ev._h)
+    def make(n_layers, score_tensor=None, config=cfg):
+        ev = pkg.Evictor(config, bs, n_layers, 7, max_sequences=B, max_tracked_tokens=8448, device=0,
+                         stream=torch.cuda.current_stream(dev))
+        ptrs = (C.c_void_p * n_layers)(*[C.c_void_p((scores if score_tensor is None else score_tensor).data_ptr())] * n_layers)
+        counts = np.zeros(B * n_layers, np.int32)
+        blocks = np.empty(B * n_layers * 256, np.int32)
+        blocks.fill(0)  # (touched here: the first write into fresh pages is not the library's time)
 
-    def evict():
-        L.check(lib.pa_evictor_evict(ev._h, B, p32(slots), p32(counts), p32(blocks), 256), lib.pa_evictor_last_error, ev._h)
+        def register(offsets):
+            L.check(lib.pa_evictor_register_scores(ev._h, B, p32(slots), ptrs, p64(offsets), None), lib.pa_evictor_last_error, ev._h)
+
+        pool = {}
+
+        def diversity():  # [n / bs, n] floats per sequence for the eviction that is due, the same tensor for every layer
+            rb_, re_ = ev.get_evictable_block_range(0, 0)
+            n_evictable = (re_ - rb_) * bs
+            per = (n_evictable // bs) * n_evictable
+            if pool.get("n", 0) < B * per:
+                pool["t"] = -torch.rand(B * per, device=dev, dtype=torch.float32)
+                pool["n"] = B * per
+            off = (np.arange(B + 1, dtype=np.int64) * per)
+            dp = (C.c_void_p * n_layers)(*[C.c_void_p(pool["t"].data_ptr())] * n_layers)
+            return pool["t"], off, dp
+
+        def register_diversity(d):
+            L.check(lib.pa_evictor_register_block_diversity(ev._h, B, p32(slots), d[2], p64(d[1])), lib.pa_evictor_last_error, ev._h)
+
+        def evict():
+            L.check(lib.pa_evictor_evict(ev._h, B, p32(slots), p32(counts), p32(blocks), 256), lib.pa_evictor_last_error, ev._h)
+
+        return ev, register, diversity, register_diversity, evict, counts
 
     kv = spec["past_lens"].astype(np.int64) + 1
     offsets = np.concatenate([[0], np.cumsum(kv)]).astype(np.int64)
@@ -182,43 +216,97 @@ def eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, layers):
     # the first launch of a kernel also loads its code: a throw-away evictor takes that
     warm = pkg.Evictor(cfg, bs, 1, 7, max_sequences=1, max_tracked_tokens=8448, device=0, stream=torch.cuda.current_stream(dev))
     warm.register_new_token_scores([0], [scores.data_ptr()], [0, 2000], None)
+    if rkv:
+        n0 = (2000 - start - 128) // bs * bs
+        wd = -torch.rand((n0 // bs) * n0, device=dev, dtype=torch.float32)
+        warm.register_block_diversity([0], [wd.data_ptr()], [0, wd.numel()])
     warm.evict_logical_blocks([0], max_blocks_per_entry=256)
     del warm
     torch.cuda.synchronize(dev)
+    # ---- first registration + eviction over the whole context
+    first_layers = min(layers, 2) if rkv else layers
+    ev, register, diversity, register_diversity, evict, counts = make(first_layers)
     t0 = time.perf_counter()
     register(offsets)
     torch.cuda.synchronize(dev)
     t1 = time.perf_counter()
+    t_div = 0.0
+    d = None
+    if rkv:
+        d = diversity()
+        torch.cuda.synchronize(dev)
+        a = time.perf_counter()
+        register_diversity(d)
+        torch.cuda.synchronize(dev)
+        t_div = time.perf_counter() - a
+        t1 = time.perf_counter()
     evict()
     torch.cuda.synchronize(dev)
     t2 = time.perf_counter()
     first_counts = counts.copy()
-    tracked = int((kv - 32).sum()) * layers
-    # steady state: one more token per sequence on a 1024-token cache (scores of the capped context)
-    kv2 = np.full(B, 1056 - 32 + 1 + 32, np.int64)
-    reg, evi, both = [], [], []
-    for _ in range(12):
-        off2 = np.concatenate([[0], np.cumsum(kv2)]).astype(np.int64)
+    tracked = int((kv - 32).sum()) * first_layers
+    d = None
+    del ev
+    t_distinct = None
+    if mode == "kvcrush":
+        # KVCrush marks the better half of the tokens; where that half ends inside a run of equal scores the choice
+        # is the host sorting routine's and the library walks that entry's scores on the host (threads).  This
+        # synthetic workload's scores underflow to exactly 0 for most of the context; uniform random scores still tie,
+        # because max pooling (window 7, the pipeline's) repeats a local maximum over its neighbours.  With a budget
+        # of 8 the steady state's one block per step is below the budget and nothing is thinned; `_budget_1` is the
+        # steady state where every eviction is.
+        distinct = torch.rand(scores.numel(), device=dev, dtype=torch.float32)
+        ev, register, diversity, register_diversity, evict, counts = make(first_layers, distinct)
+        register(offsets)
+        torch.cuda.synchronize(dev)
         a = time.perf_counter()
-        register(off2)
-        b_ = time.perf_counter()   # (the registration is left in flight: the eviction follows on the same stream)
         evict()
-        c_ = time.perf_counter()
-        reg.append(b_ - a)
-        evi.append(c_ - b_)
-        both.append(c_ - a)
-        kv2 = kv2 + 1
-    torch.cuda.synchronize(dev)
-    return {"layers": layers, "sequences": B,
-            "first_register_ms": round((t1 - t0) * 1e3, 3), "first_evict_ms": round((t2 - t1) * 1e3, 3),
-            "first_register_GBps": round(tracked * 20 / (t1 - t0) / 1e9, 1),
+        t_distinct = time.perf_counter() - a
+        del ev, distinct
+    # ---- steady state: a block of new tokens per sequence on a 1024-token cache (scores of the capped context)
+    def steady(config):
+        ev, register, diversity, register_diversity, evict, counts = make(layers, None, config)
+        kv2 = np.full(B, 1024, np.int64)
+        register(np.concatenate([[0], np.cumsum(kv2)]).astype(np.int64))  # (brings the slots to the capped length, untimed)
+        torch.cuda.synchronize(dev)
+        kv2 = kv2 + 33
+        reg, evi, both, most = [], [], [], []
+        for _ in range(12):
+            off2 = np.concatenate([[0], np.cumsum(kv2)]).astype(np.int64)
+            a = time.perf_counter()
+            register(off2)
+            if rkv:
+                register_diversity(diversity())
+            b_ = time.perf_counter()   # (the registration is left in flight: the eviction follows on the same stream)
+            evict()
+            c_ = time.perf_counter()
+            reg.append(b_ - a)
+            evi.append(c_ - b_)
+            both.append(c_ - a)
+            most.append(int(counts.max()))
+            # what stays: a retained representative makes the next eviction take two blocks
+            kv2 = kv2 - counts.reshape(B, layers)[:, 0].astype(np.int64) * bs + bs  # a block of new tokens per step
+        torch.cuda.synchronize(dev)
+        return reg, evi, both, most
+
+    reg, evi, both, steady_counts = steady(cfg)
+    every = steady(cfg_every) if mode == "kvcrush" else None
+    return {"mode": mode, "layers": layers, "sequences": B, "first_eviction_layers": first_layers,
+            "first_register_ms": round((t1 - t0 - t_div) * 1e3, 3), "first_evict_ms": round((t2 - t1) * 1e3, 3),
+            "first_register_diversity_ms": round(t_div * 1e3, 3) if rkv else None,
+            "first_evict_ms_uniform_random_scores": round(t_distinct * 1e3, 3) if t_distinct is not None else None,
+            "steady_evict_call_ms_budget_1": round(float(np.median(every[1])) * 1e3, 3) if every else None,
+            "steady_register_plus_evict_ms_budget_1": round(float(np.median(every[2])) * 1e3, 3) if every else None,
+            "first_register_GBps": round(tracked * 20 / (t1 - t0 - t_div) / 1e9, 1),
             "blocks_evicted_per_sequence_and_layer_first": [int(first_counts.min()), int(first_counts.max())],
+            "blocks_evicted_per_entry_steady_max": steady_counts,
             "steady_register_call_ms": round(float(np.median(reg)) * 1e3, 3),
             "steady_evict_call_ms": round(float(np.median(evi)) * 1e3, 3),
             "steady_register_plus_evict_ms": round(float(np.median(both)) * 1e3, 3),
             "note": "host wall clock per C-ABI call, %d sequences x %d layers per call; the steady-state pair is timed "
                     "as one (register returns with its kernel in flight, evict returns with the block lists on the "
-                    "host); first_register_GBps prices 20 bytes per tracked token (4 read, 16 written)" % (B, layers)}
+                    "host; ADAPTIVE_RKV: the registration of the diversity matrices counts as registration); "
+                    "first_register_GBps prices 20 bytes per tracked token (4 read, 16 written)" % (B, layers)}
 
 
 def kv_cache_leg(torch, pkg, dev, layers=32, blocks=256):
@@ -539,6 +627,8 @@ def main():
         res["kv_cache"] = kv_cache_leg(torch, pkg, dev)
     if args.config == 4:
         res["eviction"] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers)
+        for mode in [m for m in args.evict_modes.split(",") if m and m != "norm_sum"]:
+            res["eviction_" + mode] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers, mode)
     if not args.no_cpu_baseline:
         from oracle import oracle as O
         q_h = q.view(torch.int16).cpu().numpy().view(np.uint16)

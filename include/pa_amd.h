@@ -371,8 +371,9 @@ int32_t pa_evictor_register_scores(pa_evictor* ev, int32_t num_sequences, const 
 /* register_block_diversity (cache_eviction.cpp:526-541) for a batch of sequences, ADAPTIVE_RKV mode:
  * `diversity_per_layer` is a host array of num_decoder_layers device pointers
  * (`adaptive_rkv_diversity.<L>`); sequence i's [evictable / block_size, evictable] f32 matrix is
- * [offsets[i], offsets[i+1]) in each of them.  The values are copied; they are dropped by the next
- * pa_evictor_evict that names the sequence. */
+ * [offsets[i], offsets[i+1]) in each of them.  The values are copied (one launch for the whole batch, queued on
+ * the evictor's stream like pa_evictor_register_scores: the tensors are read in stream order, the host arrays are
+ * free on return); they are dropped by the next pa_evictor_evict that names the sequence. */
 int32_t pa_evictor_register_block_diversity(pa_evictor* ev, int32_t num_sequences, const int32_t* slots,
                                             const float* const* diversity_per_layer, const int64_t* offsets);
 /* evict_logical_blocks for a batch of sequences.  counts[i*L + l] = blocks evicted for sequence i,

@@ -20,11 +20,14 @@
 // All arithmetic is IEEE binary64 / integer in a fixed order, so results match a scalar CPU
 // evaluation bit for bit.  HBM-bound: every tracked entry is read and written once per call.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
+#include <exception>
 #include <set>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/pa_amd.h"
@@ -303,8 +306,132 @@ struct GatherEntry {
 };
 __global__ __launch_bounds__(256) void evict_gather_kernel(const GatherEntry* __restrict__ entries,
                                                            const double* __restrict__ scores, double* __restrict__ out) {
-    const GatherEntry e = entries[blockIdx.y];
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < e.n; i += gridDim.x * 256) out[e.dst_off + i] = scores[e.state_off + i];
+    const GatherEntry e = entries[blockIdx.x];
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < e.n; i += gridDim.y * 256) out[e.dst_off + i] = scores[e.state_off + i];
+}
+
+// Copies of float vectors between device buffers, all of a call in one launch (blockIdx.x = vector, .y = its part).
+struct CopyEntry {
+    const float* src;
+    float* dst;
+    int64_t n;
+};
+__global__ __launch_bounds__(256) void evict_copy_kernel(const CopyEntry* __restrict__ entries) {
+    const CopyEntry e = entries[blockIdx.x];
+    const int64_t step = (int64_t)gridDim.y * 256, first = (int64_t)blockIdx.y * 256 + threadIdx.x;
+    if ((((uintptr_t)e.src | (uintptr_t)e.dst) & 15) == 0) {
+        const float4* s4 = reinterpret_cast<const float4*>(e.src);
+        float4* d4 = reinterpret_cast<float4*>(e.dst);
+        const int64_t n4 = e.n / 4;
+        for (int64_t i = first; i < n4; i += step) d4[i] = s4[i];
+        for (int64_t i = n4 * 4 + first; i < e.n; i += step) e.dst[i] = e.src[i];
+    } else {
+        for (int64_t i = first; i < e.n; i += step) e.dst[i] = e.src[i];
+    }
+}
+
+// KVCrush on the device (kvcrush.cpp:14-111), one workgroup per (sequence, layer) whose chosen blocks are thinned:
+// the indicator bit of every token of the evictable area (1 for the half with the larger scores), the anchor point,
+// and per block the Hamming distance between its bits and the anchor -- everything that walks tokens.  The host is
+// left with one distance per block for the choice of the representatives (kvcrush.cpp:113-148, a std::sort whose
+// order among equal distances is part of the contract).
+// The reference picks the top half with std::partial_sort, so among tokens whose score equals the half's smallest one
+// the choice is the library's: when not all of them fall on one side, `flags` says so and the host works that entry
+// through from the scores themselves.
+struct CrushEntry {
+    int64_t state_off;   // first tracked score of this (slot, layer)
+    int32_t n_tok;       // tokens of the evictable area
+    int32_t dist_off;    // first entry of the block distances in the packed output
+    int32_t anchor_off;  // first byte of this entry's anchor point (modes whose anchor the host supplies)
+    int32_t pad;
+};
+__device__ __forceinline__ uint64_t score_key(double v) {  // ascending as unsigned integers; -0.0 and +0.0 alike
+    uint64_t u = (uint64_t)__double_as_longlong(v);
+    if (u == 0x8000000000000000ull) u = 0;
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+}
+__global__ __launch_bounds__(256) void evict_crush_kernel(const CrushEntry* __restrict__ entries,
+                                                          const double* __restrict__ scores,
+                                                          const uint8_t* __restrict__ host_anchors, int32_t* __restrict__ dist,
+                                                          int32_t* __restrict__ flags, int32_t bsz, int32_t anchor_mode) {
+    __shared__ uint32_t hist[256];
+    __shared__ uint64_t s_prefix;
+    __shared__ uint32_t s_rank, s_gt, s_eq;
+    extern __shared__ uint32_t ones[];  // [bsz] indicator bits set per in-block position, then the anchor point
+    const CrushEntry e = entries[blockIdx.x];
+    const int tid = threadIdx.x, n = e.n_tok;
+    const double* sc = scores + e.state_off;
+    const int half = n / 2;
+    if (half == 0) {  // no token is marked: every bit is 0
+        if (tid == 0) flags[blockIdx.x] = 0;
+    }
+    // ---- the smallest key of the top half: ascending rank n - half, by radix selection from the top byte down
+    if (tid == 0) {
+        s_prefix = 0;
+        s_rank = (uint32_t)(n - half);
+        s_gt = 0;
+        s_eq = 0;
+    }
+    for (int pass = 7; pass >= 0 && half > 0; --pass) {
+        hist[tid] = 0;
+        __syncthreads();
+        const uint64_t hi_mask = pass == 7 ? 0ull : (~0ull << (8 * (pass + 1)));
+        const uint64_t prefix = s_prefix;
+        for (int i = tid; i < n; i += 256) {
+            const uint64_t k = score_key(sc[i]);
+            if ((k & hi_mask) == (prefix & hi_mask)) atomicAdd(&hist[(k >> (8 * pass)) & 255], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t cum = 0, rank = s_rank;
+            int b = 0;
+            for (; b < 255; ++b) {
+                if (cum + hist[b] > rank) break;
+                cum += hist[b];
+            }
+            s_rank = rank - cum;
+            s_prefix = prefix | ((uint64_t)b << (8 * pass));
+        }
+        __syncthreads();
+    }
+    const uint64_t thr = s_prefix;
+    if (half > 0) {
+        uint32_t gt = 0, eq = 0;
+        for (int i = tid; i < n; i += 256) {
+            const uint64_t k = score_key(sc[i]);
+            gt += k > thr;
+            eq += k == thr;
+        }
+        atomicAdd(&s_gt, gt);
+        atomicAdd(&s_eq, eq);
+        __syncthreads();
+        // all tokens at the threshold belong to the half, or the choice among them is the sorting routine's
+        if (tid == 0) flags[blockIdx.x] = (s_eq == (uint32_t)half - s_gt) ? 0 : 1;
+    }
+    auto bit = [&](int i) -> uint32_t { return half > 0 && score_key(sc[i]) >= thr ? 1u : 0u; };
+    // ---- the anchor point: bsz bits in `ones`
+    const int blocks = n / bsz;
+    for (int j = tid; j < bsz; j += 256) ones[j] = 0;
+    __syncthreads();
+    if (anchor_mode == pa::ANCHOR_MEAN) {  // majority bit per in-block position (kvcrush.cpp:57-69)
+        for (int i = tid; i < blocks * bsz; i += 256)
+            if (bit(i)) atomicAdd(&ones[i % bsz], 1u);
+        __syncthreads();
+        for (int j = tid; j < bsz; j += 256) ones[j] = 2 * ones[j] > (uint32_t)blocks ? 1u : 0u;
+    } else {
+        for (int j = tid; j < bsz; j += 256)
+            ones[j] = anchor_mode == pa::ANCHOR_ZEROS ? 0u : anchor_mode == pa::ANCHOR_ONES ? 1u
+                    : anchor_mode == pa::ANCHOR_ALTERNATING ? (uint32_t)(j & 1) : (uint32_t)host_anchors[e.anchor_off + j];
+    }
+    __syncthreads();
+    // ---- Hamming distance of every block's bits to the anchor (kvcrush.cpp:84-111): a wave per block
+    const int lane = tid & 63, wv = tid >> 6;
+    for (int b = wv; b < blocks; b += 4) {
+        uint32_t d = 0;
+        for (int j = lane; j < bsz; j += 64) d += bit(b * bsz + j) != ones[j];
+        for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        if (lane == 0) dist[e.dist_off + b] = (int32_t)d;
+    }
 }
 
 constexpr int RKV_MAX_WINDOW = 32;
@@ -383,8 +510,8 @@ __global__ __launch_bounds__(256) void evict_filtered_diversity_kernel(const Fil
 #pragma clang fp contract(off)
     __shared__ double part[256];
     __shared__ int32_t has[256];
-    const FiltEntry e = entries[blockIdx.y];
-    const int row = blockIdx.x;
+    const FiltEntry e = entries[blockIdx.x];
+    const int row = blockIdx.y;
     if (row >= e.n_blocks) return;
     const float* r = e.div + (int64_t)row * e.n_blocks * bsz;
     const int32_t* flag = in_set + e.list_off;
@@ -463,7 +590,7 @@ struct pa_evictor {
     unsigned long long* counters = nullptr;
     std::vector<uint64_t> len;          // [slot * L + layer]
     std::vector<uint64_t> snapkv_seen;  // [slot]
-    DevBuf d_entries, d_ptrs, d_bscore, d_flags, d_list, d_filt, d_gather, d_gather_entries;
+    DevBuf d_entries, d_ptrs, d_bscore, d_flags, d_list, d_filt, d_gather, d_gather_entries, d_copies;
     // pinned host staging: one buffer for what a call uploads, one for what it reads back; `staged` marks the end
     // of the last upload from h_up (the buffer may be refilled once it has passed)
     PinnedBuf h_up, h_back;
@@ -603,8 +730,10 @@ pa_evictor* make(const pa_evictor_config* cfg, bool areas, uint64_t ignore_block
         ev->h_up.reserve(up);
         ev->d_entries.reserve(pairs * std::max(sizeof(RegEntry), sizeof(SelEntry)));
         ev->d_ptrs.reserve((size_t)cfg->num_decoder_layers * sizeof(float*));
-        ev->d_list.reserve(pairs * sizeof(int32_t));
-        ev->h_back.reserve(pairs * sizeof(int32_t));
+        // (block lists of a whole-context eviction of every pair: 1 / (4 * block_size) of the tracked scores' size)
+        const size_t lists = pairs * std::max<size_t>(1, (size_t)(cfg->max_tracked_tokens / cfg->block_size)) * sizeof(int32_t);
+        ev->d_list.reserve(lists);
+        ev->h_back.reserve(lists);
     } catch (...) {
         (void)hipFree(ev->scores);
         (void)hipFree(ev->counters);
@@ -630,6 +759,31 @@ pa_evictor* make(const pa_evictor_config* cfg, bool areas, uint64_t ignore_block
     for (auto& c : ev->crush)
         c.init(cfg->kvcrush_budget, cfg->kvcrush_anchor_point_mode, cfg->kvcrush_rng_seed, cfg->block_size);
     return ev;
+}
+
+// Runs fn(0..count-1) over up to 16 host threads (the items must be independent); the first failure of any of them is
+// rethrown after all have ended.
+template <typename F>
+void parallel_items(size_t count, size_t n_threads, F&& fn) {
+    n_threads = std::min<size_t>({n_threads, count, 16, std::max(1u, std::thread::hardware_concurrency())});
+    if (n_threads <= 1) {
+        for (size_t i = 0; i < count; ++i) fn(i);
+        return;
+    }
+    std::atomic<size_t> next{0};
+    std::atomic<bool> failed{false};
+    std::exception_ptr failure;
+    std::vector<std::thread> pool;
+    for (size_t t = 0; t < n_threads; ++t)
+        pool.emplace_back([&] {
+            try {
+                for (size_t i = next.fetch_add(1); i < count && !failed; i = next.fetch_add(1)) fn(i);
+            } catch (...) {
+                if (!failed.exchange(true)) failure = std::current_exception();
+            }
+        });
+    for (std::thread& t : pool) t.join();
+    if (failed) std::rethrow_exception(failure);
 }
 
 void upload(pa_evictor* ev, DevBuf& buf, const void* src, size_t bytes) {
@@ -789,6 +943,7 @@ void pa_evictor_destroy(pa_evictor* ev) {
     if (ev->hist) (void)hipFree(ev->hist);
     for (auto& b : ev->div_buf) b.release();
     ev->d_filt.release();
+    ev->d_copies.release();
     ev->d_entries.release();
     ev->d_ptrs.release();
     ev->d_bscore.release();
@@ -930,21 +1085,32 @@ int32_t pa_evictor_register_block_diversity(pa_evictor* ev, int32_t B, const int
                        "diversity size must be a multiple of the block size");
         }
         HIP_CHECK(hipSetDevice(ev->cfg.device));
+        // one launch copies every (sequence, layer) matrix; the per-sequence buffers only ever grow
+        const size_t bytes = (size_t)B * L * sizeof(CopyEntry);
+        CopyEntry* copies = reinterpret_cast<CopyEntry*>(stage_begin(ev, bytes));
+        int64_t longest = 0;
         for (int32_t i = 0; i < B; ++i) {
             const uint64_t n = (uint64_t)(offsets[i + 1] - offsets[i]);
             DevBuf& buf = ev->div_buf[slots[i]];
             buf.reserve(std::max<uint64_t>(1, n * L) * sizeof(float));
-            std::vector<uint64_t> off(L + 1);
-            for (uint64_t l = 0; l < L; ++l) {
-                off[l] = l * n;
-                if (n)
-                    HIP_CHECK(hipMemcpyAsync(buf.as<float>() + off[l], diversity_per_layer[l] + offsets[i], n * sizeof(float),
-                                             hipMemcpyDeviceToDevice, ev->stream));
-            }
-            off[L] = L * n;
-            ev->div_off[slots[i]] = off;
+            for (uint64_t l = 0; l < L; ++l)
+                copies[(size_t)i * L + l] = CopyEntry{diversity_per_layer[l] + offsets[i], buf.as<float>() + l * n, (int64_t)n};
+            longest = std::max<int64_t>(longest, (int64_t)n);
         }
-        HIP_CHECK(hipStreamSynchronize(ev->stream));
+        if (longest > 0) {
+            stage_copy(ev, ev->d_copies, 0, bytes);
+            stage_end(ev);
+            const unsigned gx = (unsigned)std::max<int64_t>(1, std::min<int64_t>((longest + 4095) / 4096, 256));
+            hipLaunchKernelGGL(evict_copy_kernel, dim3((unsigned)((size_t)B * L), gx), dim3(256), 0, ev->stream,
+                               ev->d_copies.as<CopyEntry>());
+            HIP_CHECK(hipGetLastError());
+        }
+        for (int32_t i = 0; i < B; ++i) {
+            const uint64_t n = (uint64_t)(offsets[i + 1] - offsets[i]);
+            std::vector<uint64_t>& off = ev->div_off[slots[i]];
+            off.resize(L + 1);
+            for (uint64_t l = 0; l <= L; ++l) off[l] = l * n;
+        }
     });
 }
 
@@ -956,7 +1122,7 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
         PA_REQUIRE(ev->has_areas, PA_PARAMETER_MISMATCH, "a bare score manager has no eviction areas");
         const uint64_t L = ev->L(), bsz = ev->cfg.block_size;
         const bool rkv = ev->rkv();
-        const bool crush = !rkv && ev->cfg.kvcrush_budget > 0;
+        bool crush = !rkv && ev->cfg.kvcrush_budget > 0;  // (below: and only where enough blocks are chosen)
         std::vector<SelEntry> entries((size_t)B * L);
         int64_t list_total = 0, k_total = 0;
         int32_t most_blocks_any = 0, most_k = 0;
@@ -1012,6 +1178,10 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             finish(nullptr, false);
             return;
         }
+        if (crush) {  // cache_eviction.cpp:365-366: representatives stay only where at least `budget` blocks were chosen
+            crush = false;
+            for (const SelEntry& e : entries) crush = crush || (e.k > 0 && (uint64_t)e.k >= ev->cfg.kvcrush_budget);
+        }
         HIP_CHECK(hipSetDevice(ev->cfg.device));
         const int32_t norm = ev->cfg.aggregation_mode == PA_AGG_NORM_SUM ? 1 : 0;
         const size_t fused_lds = select_lds_bytes(most_blocks_any, (int64_t)bsz, most_k);
@@ -1058,29 +1228,32 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             std::vector<size_t> left(entries.size(), 0);
             std::vector<int32_t> in_set((size_t)list_total, 0);
             std::vector<FiltEntry> filt;
-            std::vector<size_t> filt_entry;
             int32_t most_blocks = 0;
-            for (size_t x = 0; x < entries.size(); ++x) {
+            // (the entries are independent: host threads share the two loops over them)
+            parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
                 const SelEntry& e = entries[x];
-                if (e.n_blocks <= 0) continue;
+                if (e.n_blocks <= 0) return;
                 size_t kept = 0;
                 sets[x] = calc.diversity_block_set(max_keep, bscore.data() + e.list_off, (size_t)e.n_blocks, &kept);
                 left[x] = max_keep - kept;
-                if (left[x] == 0) continue;
+                if (left[x] == 0) return;
                 PA_REQUIRE(left[x] <= sets[x].size(), PA_GENERAL_ERROR,
                            "more blocks left to fill than the diversity set holds");
                 for (size_t b : sets[x]) in_set[(size_t)e.list_off + b] = 1;
+            });
+            for (size_t x = 0; x < entries.size(); ++x) {
+                const SelEntry& e = entries[x];
+                if (e.n_blocks <= 0 || left[x] == 0) continue;
                 const int32_t slot = slots[x / L];
                 filt.push_back(FiltEntry{ev->div_buf[slot].as<float>() + ev->div_off[slot][x % L], e.list_off, e.n_blocks,
                                          (int32_t)sets[x].size()});
-                filt_entry.push_back(x);
                 most_blocks = std::max(most_blocks, e.n_blocks);
             }
             std::vector<double> filtered((size_t)list_total, 0.0);
             if (!filt.empty()) {
                 upload(ev, ev->d_filt, filt.data(), filt.size() * sizeof(FiltEntry));
                 upload(ev, ev->d_flags, in_set.data(), in_set.size() * sizeof(int32_t));
-                hipLaunchKernelGGL(evict_filtered_diversity_kernel, dim3((unsigned)most_blocks, (unsigned)filt.size()),
+                hipLaunchKernelGGL(evict_filtered_diversity_kernel, dim3((unsigned)filt.size(), (unsigned)most_blocks),
                                    block, 0, ev->stream, ev->d_filt.as<FiltEntry>(), ev->d_flags.as<int32_t>(),
                                    ev->d_bscore.as<double>(), (int32_t)bsz);
                 HIP_CHECK(hipGetLastError());
@@ -1088,9 +1261,9 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
                                          hipMemcpyDeviceToHost, ev->stream));
                 HIP_CHECK(hipStreamSynchronize(ev->stream));
             }
-            for (size_t x = 0; x < entries.size(); ++x) {
+            parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
                 SelEntry& e = entries[x];
-                if (e.n_blocks <= 0) continue;
+                if (e.n_blocks <= 0) return;
                 std::set<size_t> keep;
                 if (left[x] != 0) keep = calc.most_diverse_blocks(left[x], sets[x], filtered.data() + e.list_off);
                 int32_t k = 0;
@@ -1098,7 +1271,7 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
                     if (!keep.count(b)) lists[(size_t)e.list_off + k++] = (int32_t)b;
                 PA_REQUIRE(k <= max_per_entry, PA_OUT_OF_BOUNDS, "more evicted blocks than the output holds");
                 e.k = k;
-            }
+            });
         } else {
             hipLaunchKernelGGL(evict_rank_kernel, grid, block, 0, ev->stream, ev->d_entries.as<SelEntry>(),
                                ev->d_bscore.as<double>(), ev->d_flags.as<int32_t>());
@@ -1110,44 +1283,102 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             HIP_CHECK(hipStreamSynchronize(ev->stream));
             lists_on_device = true;
             if (crush) {  // cache_eviction.cpp:367-398: some of the chosen blocks stay as representatives
-                // the token scores of every pair that needs them come back in one packed read
-                std::vector<GatherEntry> gather;
-                std::vector<size_t> gather_of(entries.size(), SIZE_MAX);
-                int64_t packed = 0;
-                int32_t longest = 0;
+                // Everything that walks tokens runs on the device (evict_crush_kernel); one distance per block comes
+                // back.  Anchor points that do not depend on the scores are made here, in the order the reference
+                // makes them (one per thinned entry, entries in call order: the random mode draws from the
+                // sequence's generator), and go up with the entries.
+                const int32_t mode = ev->cfg.kvcrush_anchor_point_mode;
+                std::vector<CrushEntry> work;
+                std::vector<size_t> work_entry;
+                std::vector<uint8_t> anchors;
+                int64_t dist_total = 0;
                 for (size_t x = 0; x < entries.size(); ++x) {
                     const SelEntry& e = entries[x];
                     if (e.k <= 0 || (uint64_t)e.k < ev->cfg.kvcrush_budget) continue;
-                    gather_of[x] = gather.size();
-                    gather.push_back(GatherEntry{e.state_off, packed, (int32_t)((size_t)e.n_blocks * bsz), 0});
-                    packed += (int64_t)e.n_blocks * (int64_t)bsz;
-                    longest = std::max(longest, gather.back().n);
+                    CrushEntry w{e.state_off, (int32_t)((size_t)e.n_blocks * bsz), (int32_t)dist_total, (int32_t)anchors.size(), 0};
+                    if (mode != pa::ANCHOR_MEAN) {
+                        std::vector<uint8_t> anchor;
+                        PA_REQUIRE(ev->crush[slots[x / L]].anchor_point((size_t)w.n_tok, nullptr, anchor), PA_PARAMETER_MISMATCH,
+                                   "Invalid anchor point type");
+                        anchors.insert(anchors.end(), anchor.begin(), anchor.end());
+                    }
+                    work.push_back(w);
+                    work_entry.push_back(x);
+                    dist_total += e.n_blocks;
+                    PA_REQUIRE(dist_total <= INT32_MAX, PA_OUT_OF_BOUNDS, "too many evictable blocks for one call");
                 }
-                if (!gather.empty()) {
-                    upload(ev, ev->d_gather_entries, gather.data(), gather.size() * sizeof(GatherEntry));
-                    ev->d_gather.reserve((size_t)packed * sizeof(double));
-                    ev->h_back.reserve((size_t)packed * sizeof(double));
-                    hipLaunchKernelGGL(evict_gather_kernel, dim3((unsigned)std::min(pa::ceil_div(longest, 256), 32), (unsigned)gather.size()),
-                                       dim3(256), 0, ev->stream, ev->d_gather_entries.as<GatherEntry>(), ev->scores,
-                                       ev->d_gather.as<double>());
+                if (!work.empty()) {
+                    upload(ev, ev->d_gather_entries, work.data(), work.size() * sizeof(CrushEntry));
+                    if (!anchors.empty()) upload(ev, ev->d_filt, anchors.data(), anchors.size());
+                    // distances, then one flag per entry
+                    const size_t back_ints = (size_t)dist_total + work.size();
+                    ev->d_gather.reserve(back_ints * sizeof(int32_t));
+                    ev->h_back.reserve(back_ints * sizeof(int32_t));
+                    int32_t* d_dist = ev->d_gather.as<int32_t>();
+                    hipLaunchKernelGGL(evict_crush_kernel, dim3((unsigned)work.size()), dim3(256), (size_t)bsz * sizeof(uint32_t),
+                                       ev->stream, ev->d_gather_entries.as<CrushEntry>(), ev->scores,
+                                       ev->d_filt.as<uint8_t>(), d_dist, d_dist + dist_total, (int32_t)bsz, mode);
                     HIP_CHECK(hipGetLastError());
-                    HIP_CHECK(hipMemcpyAsync(ev->h_back.p, ev->d_gather.p, (size_t)packed * sizeof(double), hipMemcpyDeviceToHost,
+                    HIP_CHECK(hipMemcpyAsync(ev->h_back.p, ev->d_gather.p, back_ints * sizeof(int32_t), hipMemcpyDeviceToHost,
                                              ev->stream));
                     HIP_CHECK(hipStreamSynchronize(ev->stream));
-                }
-                for (size_t x = 0; x < entries.size(); ++x) {
-                    SelEntry& e = entries[x];
-                    if (gather_of[x] == SIZE_MAX) continue;
-                    const size_t n_tok = (size_t)e.n_blocks * bsz;
-                    const double* tok_data = ev->h_back.as<double>() + gather[gather_of[x]].dst_off;
-                    int32_t* list = lists.data() + e.list_off;
-                    const std::vector<size_t> chosen(list, list + e.k);
-                    const std::vector<size_t> stay = ev->crush[slots[x / L]].blocks_to_retain(n_tok, chosen, tok_data);
-                    int32_t k = 0;
-                    for (size_t b : chosen)
-                        if (std::find(stay.begin(), stay.end(), b) == stay.end()) list[k++] = (int32_t)b;
-                    if (k != e.k) lists_on_device = false;
-                    e.k = k;
+                    std::vector<int32_t> back(ev->h_back.as<int32_t>(), ev->h_back.as<int32_t>() + back_ints);
+                    // entries whose top half is not settled by the scores alone: their token scores come back and the
+                    // host walks them (same anchor point: the one made above, or the majority of the host's bits)
+                    std::vector<GatherEntry> gather;
+                    std::vector<size_t> gather_work;
+                    int64_t packed = 0;
+                    int32_t longest = 0;
+                    for (size_t w = 0; w < work.size(); ++w) {
+                        if (back[(size_t)dist_total + w] == 0) continue;
+                        gather_work.push_back(w);
+                        gather.push_back(GatherEntry{work[w].state_off, packed, work[w].n_tok, 0});
+                        packed += work[w].n_tok;
+                        longest = std::max(longest, work[w].n_tok);
+                    }
+                    if (!gather.empty()) {
+                        upload(ev, ev->d_gather_entries, gather.data(), gather.size() * sizeof(GatherEntry));
+                        ev->d_gather.reserve((size_t)packed * sizeof(double));
+                        ev->h_back.reserve((size_t)packed * sizeof(double));
+                        hipLaunchKernelGGL(evict_gather_kernel, dim3((unsigned)gather.size(), (unsigned)std::min(pa::ceil_div(longest, 256), 32)),
+                                           dim3(256), 0, ev->stream, ev->d_gather_entries.as<GatherEntry>(), ev->scores,
+                                           ev->d_gather.as<double>());
+                        HIP_CHECK(hipGetLastError());
+                        HIP_CHECK(hipMemcpyAsync(ev->h_back.p, ev->d_gather.p, (size_t)packed * sizeof(double), hipMemcpyDeviceToHost,
+                                                 ev->stream));
+                        HIP_CHECK(hipStreamSynchronize(ev->stream));
+                        // (entries are independent and nothing below touches a selector's generator: host threads share them)
+                        const double* tok_scores = ev->h_back.as<const double>();
+                        auto walk = [&](size_t g) {
+                            const size_t w = gather_work[g];
+                            pa::KvCrushSelector& sel = ev->crush[slots[work_entry[w] / L]];
+                            const size_t n_tok = (size_t)work[w].n_tok;
+                            const std::vector<uint8_t> bits = sel.indicators(n_tok, tok_scores + gather[g].dst_off);
+                            std::vector<uint8_t> anchor;
+                            if (mode == pa::ANCHOR_MEAN) (void)sel.anchor_point(n_tok, bits.data(), anchor);
+                            else anchor.assign(anchors.begin() + work[w].anchor_off, anchors.begin() + work[w].anchor_off + (long)bsz);
+                            const std::vector<size_t> d = sel.hamming(n_tok, bits.data(), anchor.data());
+                            for (size_t bidx = 0; bidx < d.size(); ++bidx) back[(size_t)work[w].dist_off + bidx] = (int32_t)d[bidx];
+                        };
+                        parallel_items(gather.size(), (size_t)(packed / 65536 + 1), walk);
+                    }
+                    // the representatives: a sort of each entry's chosen blocks by distance, entries independent
+                    std::atomic<bool> shortened{false};
+                    parallel_items(work.size(), work.size() / 64 + 1, [&](size_t w) {
+                        SelEntry& e = entries[work_entry[w]];
+                        int32_t* list = lists.data() + e.list_off;
+                        const std::vector<size_t> chosen(list, list + e.k);
+                        const std::vector<size_t> dist(back.begin() + work[w].dist_off, back.begin() + work[w].dist_off + e.n_blocks);
+                        const std::vector<size_t> stay = ev->crush[slots[work_entry[w] / L]].representative(dist.data(), dist.size(), chosen);
+                        std::vector<uint8_t> stays((size_t)e.n_blocks, 0);
+                        for (size_t b : stay) stays[b] = 1;
+                        int32_t k = 0;
+                        for (size_t b : chosen)
+                            if (!stays[b]) list[k++] = (int32_t)b;
+                        if (k != e.k) shortened = true;
+                        e.k = k;
+                    });
+                    if (shortened) lists_on_device = false;
                 }
             }
         }

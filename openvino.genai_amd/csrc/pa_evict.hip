@@ -32,6 +32,7 @@
 
 #include "../../include/pa_amd.h"
 #include "pa_device.h"
+#include "host_parallel.h"
 #include "pa_select.h"
 
 namespace {
@@ -762,31 +763,6 @@ pa_evictor* make(const pa_evictor_config* cfg, bool areas, uint64_t ignore_block
     return ev;
 }
 
-// Runs fn(0..count-1) over up to 16 host threads (the items must be independent); the first failure of any of them is
-// rethrown after all have ended.
-template <typename F>
-void parallel_items(size_t count, size_t n_threads, F&& fn) {
-    n_threads = std::min<size_t>({n_threads, count, 16, std::max(1u, std::thread::hardware_concurrency())});
-    if (n_threads <= 1) {
-        for (size_t i = 0; i < count; ++i) fn(i);
-        return;
-    }
-    std::atomic<size_t> next{0};
-    std::atomic<bool> failed{false};
-    std::exception_ptr failure;
-    std::vector<std::thread> pool;
-    for (size_t t = 0; t < n_threads; ++t)
-        pool.emplace_back([&] {
-            try {
-                for (size_t i = next.fetch_add(1); i < count && !failed; i = next.fetch_add(1)) fn(i);
-            } catch (...) {
-                if (!failed.exchange(true)) failure = std::current_exception();
-            }
-        });
-    for (std::thread& t : pool) t.join();
-    if (failed) std::rethrow_exception(failure);
-}
-
 void upload(pa_evictor* ev, DevBuf& buf, const void* src, size_t bytes) {
     buf.reserve(bytes);
     HIP_CHECK(hipMemcpyAsync(buf.p, src, bytes, hipMemcpyHostToDevice, ev->stream));
@@ -1231,7 +1207,7 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
             std::vector<FiltEntry> filt;
             int32_t most_blocks = 0;
             // (the entries are independent: host threads share the two loops over them)
-            parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
+            pa::parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
                 const SelEntry& e = entries[x];
                 if (e.n_blocks <= 0) return;
                 size_t kept = 0;
@@ -1262,7 +1238,7 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
                                          hipMemcpyDeviceToHost, ev->stream));
                 HIP_CHECK(hipStreamSynchronize(ev->stream));
             }
-            parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
+            pa::parallel_items(entries.size(), entries.size() / 64 + 1, [&](size_t x) {
                 SelEntry& e = entries[x];
                 if (e.n_blocks <= 0) return;
                 std::set<size_t> keep;
@@ -1361,11 +1337,11 @@ int32_t pa_evictor_evict(pa_evictor* ev, int32_t B, const int32_t* slots, int32_
                             const std::vector<size_t> d = sel.hamming(n_tok, bits.data(), anchor.data());
                             for (size_t bidx = 0; bidx < d.size(); ++bidx) back[(size_t)work[w].dist_off + bidx] = (int32_t)d[bidx];
                         };
-                        parallel_items(gather.size(), (size_t)(packed / 65536 + 1), walk);
+                        pa::parallel_items(gather.size(), (size_t)(packed / 65536 + 1), walk);
                     }
                     // the representatives: a sort of each entry's chosen blocks by distance, entries independent
                     std::atomic<bool> shortened{false};
-                    parallel_items(work.size(), work.size() / 64 + 1, [&](size_t w) {
+                    pa::parallel_items(work.size(), work.size() / 64 + 1, [&](size_t w) {
                         SelEntry& e = entries[work_entry[w]];
                         int32_t* list = lists.data() + e.list_off;
                         const std::vector<size_t> chosen(list, list + e.k);

@@ -11,6 +11,7 @@
 
 #include "../../include/pa_amd.h"
 #include "pa_device.h"
+#include "host_parallel.h"
 
 namespace {
 
@@ -182,6 +183,8 @@ struct pa_ctx {
     pa::StepDev dev{};
     // block tables: shared (index 0 of `tables` when shared) or per layer
     std::vector<DevBuf> tables;
+    std::vector<const void*> table_ptr;  // where each table lives: its own buffer, or a slice of table_pool
+    DevBuf table_pool;                   // the tables of a whole-model call, one after the other
     std::vector<int32_t> table_count;
     std::vector<int64_t> table_bound;  // largest block id of each table + 1: the smallest cache it may be used with
     // u8 decode kernel: its split-K plan without / with scores (fixed per step) and, behind every table, the
@@ -263,9 +266,9 @@ bool tuned_append_shape(const pa_config& c) { return kv_alike(c) && (c.head_size
 const int32_t* table_for(pa_ctx* ctx, int32_t layer) {
     PA_REQUIRE(layer >= 0 && layer < ctx->cfg.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
     const size_t idx = ctx->shared_table ? 0 : (size_t)layer;
-    PA_REQUIRE(idx < ctx->tables.size() && ctx->table_count[idx] == ctx->total_block_ids && ctx->tables[idx].p,
+    PA_REQUIRE(idx < ctx->tables.size() && ctx->table_count[idx] == ctx->total_block_ids && ctx->table_ptr[idx],
                PA_PARAMETER_MISMATCH, "block_indices for this layer were not set for the current step");
-    return ctx->tables[idx].as<int32_t>();
+    return static_cast<const int32_t*>(ctx->table_ptr[idx]);
 }
 
 void check_io(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool need_kv, bool need_q) {
@@ -953,6 +956,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->meta.release();
     ctx->items.release();
     for (auto& t : ctx->tables) t.release();
+    ctx->table_pool.release();
     ctx->step_staging.release();
     ctx->part_acc.release();
     ctx->part_ml.release();
@@ -1082,6 +1086,56 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
     });
 }
 
+namespace {
+// Largest block id of a table + 1 after the check of every id against [0, num_blocks): through the smallest and the
+// largest one (a loop without branches, which the compiler turns into vector minima and maxima: 65792 ids take 4 us
+// instead of 39).
+int64_t checked_bound(const int32_t* ids, int32_t count, int64_t num_blocks) {
+    int32_t id_lo = INT32_MAX, id_hi = INT32_MIN;
+    for (int32_t i = 0; i < count; ++i) {
+        id_lo = std::min(id_lo, ids[i]);
+        id_hi = std::max(id_hi, ids[i]);
+    }
+    PA_REQUIRE(count == 0 || (id_lo >= 0 && id_hi < num_blocks), PA_OUT_OF_BOUNDS, "block index outside the cache");
+    return count == 0 ? 0 : (int64_t)id_hi + 1;
+}
+
+// Switches the context between one table for all layers and a table per layer.
+void shape_tables(pa_ctx* ctx, bool shared) {
+    if (!ctx->tables.empty() && shared == ctx->shared_table) return;
+    ctx->shared_table = shared;
+    const size_t n = shared ? 1 : (size_t)ctx->cfg.num_layers;
+    if (ctx->tables.size() != n) {
+        HIP_CHECK(hipStreamSynchronize(ctx->stream));
+        for (auto& t : ctx->tables) t.release();
+        ctx->tables.assign(n, DevBuf());
+        ctx->table_ptr.assign(n, nullptr);
+        ctx->table_count.assign(n, -1);
+        ctx->table_bound.assign(n, 0);
+    }
+}
+
+// Bytes of a table's upload: the ids, then (u8 decode kernel) the descriptors of its single-token sequences for the
+// plan without and the plan with scores.  Sets the descriptors' offsets.
+size_t table_upload_bytes(pa_ctx* ctx, int32_t count, size_t* id_bytes, bool* with_descs) {
+    *id_bytes = std::max<size_t>(((size_t)count * sizeof(int32_t) + 127) & ~(size_t)127, 128);
+    size_t total = *id_bytes;
+    *with_descs = decode_u8_shape(ctx->cfg) && !ctx->h_dec.empty();
+    if (*with_descs)
+        for (int w = 0; w < 2; ++w) {
+            ctx->desc_off[w] = total;
+            total += ctx->h_dec.size() * ctx->dec_plan[w].nsplit * sizeof(pa::DecodeDesc);
+        }
+    return total;
+}
+
+void fill_table_stage(const pa_ctx* ctx, const int32_t* ids, int32_t count, size_t id_bytes, bool with_descs, uint8_t* stage) {
+    std::memcpy(stage, ids, (size_t)count * sizeof(int32_t));
+    std::memset(stage + (size_t)count * sizeof(int32_t), 0, id_bytes - (size_t)count * sizeof(int32_t));
+    if (with_descs) fill_decode_descs(ctx, ids, stage);
+}
+}  // namespace
+
 int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int32_t count, int64_t num_blocks) {
     if (!ctx) return PA_INVALID_C_PARAM;
     return guarded(ctx, [&] {
@@ -1090,50 +1144,72 @@ int32_t pa_set_block_indices(pa_ctx* ctx, int32_t layer, const int32_t* ids, int
         PA_REQUIRE(layer >= -1 && layer < ctx->cfg.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
         PA_REQUIRE(count == ctx->total_block_ids, PA_PARAMETER_MISMATCH,
                    "block_indices length differs from block_indices_begins[B]");
-        // every id is checked through the smallest and the largest one (a loop without branches, which the compiler
-        // turns into vector minima and maxima: 65792 ids take 4 us instead of 39)
-        int32_t id_lo = INT32_MAX, id_hi = INT32_MIN;
-        for (int32_t i = 0; i < count; ++i) {
-            id_lo = std::min(id_lo, ids[i]);
-            id_hi = std::max(id_hi, ids[i]);
-        }
-        PA_REQUIRE(count == 0 || (id_lo >= 0 && id_hi < num_blocks), PA_OUT_OF_BOUNDS, "block index outside the cache");
-        const int64_t bound = count == 0 ? 0 : (int64_t)id_hi + 1;
-        const bool shared = layer < 0;
-        if (ctx->tables.empty() || shared != ctx->shared_table) {
-            ctx->shared_table = shared;
-            const size_t n = shared ? 1 : (size_t)ctx->cfg.num_layers;
-            if (ctx->tables.size() != n) {
-                HIP_CHECK(hipStreamSynchronize(ctx->stream));
-                for (auto& t : ctx->tables) t.release();
-                ctx->tables.assign(n, DevBuf());
-                ctx->table_count.assign(n, -1);
-                ctx->table_bound.assign(n, 0);
-            }
-        }
-        const size_t idx = shared ? 0 : (size_t)layer;
-        // one upload: the ids, then (u8 decode kernel) the descriptors of its single-token sequences for the plan
-        // without and the plan with scores
-        const size_t id_bytes = ((size_t)count * sizeof(int32_t) + 127) & ~(size_t)127;
-        size_t total = std::max<size_t>(id_bytes, 128);
-        const bool with_descs = decode_u8_shape(ctx->cfg) && !ctx->h_dec.empty();
-        if (with_descs)
-            for (int w = 0; w < 2; ++w) {
-                ctx->desc_off[w] = total;
-                total += ctx->h_dec.size() * ctx->dec_plan[w].nsplit * sizeof(pa::DecodeDesc);
-            }
+        const int64_t bound = checked_bound(ids, count, num_blocks);
+        shape_tables(ctx, layer < 0);
+        const size_t idx = layer < 0 ? 0 : (size_t)layer;
+        size_t id_bytes;
+        bool with_descs;
+        const size_t total = table_upload_bytes(ctx, count, &id_bytes, &with_descs);
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         if (ctx->tables[idx].cap < total) {  // kernels in flight may still read the buffer this would free
             HIP_CHECK(hipStreamSynchronize(ctx->stream));
             ctx->tables[idx].reserve(total);
         }
         uint8_t* stage = stage_piece(ctx, total);
-        std::memcpy(stage, ids, (size_t)count * sizeof(int32_t));
-        std::memset(stage + (size_t)count * sizeof(int32_t), 0, std::max<size_t>(id_bytes, 128) - (size_t)count * sizeof(int32_t));
-        if (with_descs) fill_decode_descs(ctx, ids, stage);
+        fill_table_stage(ctx, ids, count, id_bytes, with_descs, stage);
         HIP_CHECK(hipMemcpyAsync(ctx->tables[idx].p, stage, total, hipMemcpyHostToDevice, ctx->stream));
+        ctx->table_ptr[idx] = ctx->tables[idx].p;
         ctx->table_count[idx] = count;
         ctx->table_bound[idx] = bound;
+    });
+}
+
+int32_t pa_set_block_indices_layers(pa_ctx* ctx, int32_t first_layer, int32_t num_layers, const int32_t* const* ids_per_layer,
+                                    int32_t count, int64_t num_blocks) {
+    if (!ctx) return PA_INVALID_C_PARAM;
+    return guarded(ctx, [&] {
+        PA_REQUIRE(ctx->step_ready, PA_PARAMETER_MISMATCH, "pa_step_begin has not been called");
+        PA_REQUIRE(ids_per_layer && count >= 0 && num_layers > 0, PA_INVALID_C_PARAM, "block_indices missing");
+        PA_REQUIRE(first_layer >= 0 && num_layers <= ctx->cfg.num_layers - first_layer, PA_OUT_OF_BOUNDS, "layer out of range");
+        for (int32_t l = 0; l < num_layers; ++l) PA_REQUIRE(ids_per_layer[l], PA_INVALID_C_PARAM, "block_indices missing");
+        PA_REQUIRE(count == ctx->total_block_ids, PA_PARAMETER_MISMATCH,
+                   "block_indices length differs from block_indices_begins[B]");
+        shape_tables(ctx, false);
+        size_t id_bytes;
+        bool with_descs;
+        const size_t total = table_upload_bytes(ctx, count, &id_bytes, &with_descs);
+        const size_t stride = (total + 255) & ~(size_t)255;
+        // One pass of a few host threads over the layers checks every id and fills the layer's piece of the staging
+        // area (a table is read once, while it is in the core's cache; memory-bound host work); nothing of the
+        // context changes before every layer has passed.
+        std::vector<int64_t> bound((size_t)num_layers, 0);
+        HIP_CHECK(hipSetDevice(ctx->cfg.device));
+        uint8_t* stage = stage_piece(ctx, stride * (size_t)num_layers);
+        pa::parallel_items((size_t)num_layers, std::min<size_t>(8, (size_t)num_layers * (size_t)count / 131072 + 1), [&](size_t l) {
+            bound[l] = checked_bound(ids_per_layer[l], count, num_blocks);
+            fill_table_stage(ctx, ids_per_layer[l], count, id_bytes, with_descs, stage + l * stride);
+        });
+        if (ctx->table_pool.cap < stride * (size_t)ctx->cfg.num_layers) {
+            // kernels in flight may still read the pool this frees; tables that lived in it have to be set again
+            HIP_CHECK(hipStreamSynchronize(ctx->stream));
+            const uint8_t* old = ctx->table_pool.as<uint8_t>();
+            for (size_t i = 0; i < ctx->table_ptr.size(); ++i) {
+                const uint8_t* at = static_cast<const uint8_t*>(ctx->table_ptr[i]);
+                if (old && at >= old && at < old + ctx->table_pool.cap) {
+                    ctx->table_ptr[i] = nullptr;
+                    ctx->table_count[i] = -1;
+                }
+            }
+            ctx->table_pool.reserve(stride * (size_t)ctx->cfg.num_layers);
+        }
+        uint8_t* dst = ctx->table_pool.as<uint8_t>() + (size_t)first_layer * stride;
+        HIP_CHECK(hipMemcpyAsync(dst, stage, stride * (size_t)num_layers, hipMemcpyHostToDevice, ctx->stream));
+        for (int32_t l = 0; l < num_layers; ++l) {
+            const size_t idx = (size_t)(first_layer + l);
+            ctx->table_ptr[idx] = dst + (size_t)l * stride;
+            ctx->table_count[idx] = count;
+            ctx->table_bound[idx] = bound[(size_t)l];
+        }
     });
 }
 
@@ -1533,7 +1609,7 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         stage_upload(ctx, ctx->div_seqs.p, seqs.data(), seqs.size() * sizeof(pa::RkvDivSeq));
         pa::RkvDivArgs a{};
         a.key_cache = static_cast<const uint8_t*>(key_cache);
-        a.block_indices = ctx->tables[tidx].as<int32_t>();
+        a.block_indices = static_cast<const int32_t*>(ctx->table_ptr[tidx]);
         a.seqs = ctx->div_seqs.as<pa::RkvDivSeq>();
         a.stats = ctx->div_stats.as<float4>();
         a.mean = ctx->div_mean.as<float>();

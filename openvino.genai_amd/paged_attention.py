@@ -75,6 +75,15 @@ class PagedAttention:
         ids = _i32(block_indices)
         self._ck(L.lib().pa_set_block_indices(self._h, layer, _p32(ids), len(ids), int(num_blocks)))
 
+    def set_block_indices_per_layer(self, tables, num_blocks, first_layer=0):
+        """`block_indices.<L>` of layers first_layer .. first_layer + len(tables) - 1 in one call."""
+        arrs = [_i32(t) for t in tables]
+        n = len(arrs[0]) if arrs else 0
+        if any(len(a) != n for a in arrs):
+            raise ValueError("every layer's block_indices must have the same length")
+        ptrs = (C.POINTER(C.c_int32) * len(arrs))(*[_p32(a) for a in arrs])
+        self._ck(L.lib().pa_set_block_indices_layers(self._h, int(first_layer), len(arrs), ptrs, n, int(num_blocks)))
+
     def _io(self, query, key, value, key_cache, value_cache, out, scores):
         io = L.pa_layer_io()
         ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None

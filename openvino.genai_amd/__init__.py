@@ -10,6 +10,7 @@ from .cache_eviction import (AdaptiveRKVBlockCalculator, AdaptiveRKVConfig, Aggr
                              rotation_trig_lut, snapkv_num_token_scores_to_aggregate)
 from .kv_cache import KVCacheManager, normalize_num_kv_blocks  # noqa: F401
 from .paged_attention import PagedAttention, pack_step, row_bytes  # noqa: F401
+from .pipeline_metrics import PipelineMetrics, PipelineMetricsTracker, used_percentage  # noqa: F401
 from .scheduler_config import SchedulerConfig  # noqa: F401
 from .sparse_attention import (SparseAttentionConfig, SparseAttentionMode,  # noqa: F401
                                TriShapeSparseAttentionTokenSkipper, schedule_xattention_threshold)

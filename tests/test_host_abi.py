@@ -105,6 +105,38 @@ def test_config_surface_keeps_reference_names(pkg):
     assert "sparseAttentionMode: TRISHAPE" in sc.to_string() and "xattention_stride: 8" in sc.to_string()
 
 
+def test_pipeline_metrics_keep_reference_names_and_bookkeeping(pkg):
+    # fields: include/openvino/genai/continuous_batching_pipeline.hpp:33-75; Python names:
+    # src/python/py_continuous_batching_pipeline.cpp:461-467
+    m = pkg.PipelineMetrics()
+    for name in ("requests", "scheduled_requests", "cache_usage", "avg_cache_usage", "cache_size_in_bytes",
+                 "kv_cache_size_in_bytes", "max_cache_usage", "inference_duration", "sampling_duration"):
+        assert getattr(m, name) == 0
+    m.cache_size_in_bytes = 7
+    assert m.kv_cache_size_in_bytes == 7
+    # BlockAllocator::get_used_percentage (block_manager.hpp:588-592) in float32: 2 layers x 10 blocks, 3 + 4 free
+    assert pkg.used_percentage([3, 4], 10) == float(np.float32(13) / np.float32(20) * np.float32(100)) == 65.0
+    assert pkg.used_percentage([10, 10], 10) == 0.0 and pkg.used_percentage([0], 3) == 100.0
+    t = pkg.PipelineMetricsTracker()
+    usages = []
+    for step in range(1200):                    # pipeline_impl.cpp:394-398 with the 1000-step window of :779-789
+        free = [step % 7, (3 * step) % 11]
+        usages.append(t.register_step(free, 16, requests=5, scheduled_requests=3, cache_size_in_bytes=1 << 20))
+        got = t.get_metrics()
+        assert got.cache_usage == usages[-1] and got.max_cache_usage == max(usages)
+        assert got.avg_cache_usage == float(np.float32(sum(usages[-1000:]) / len(usages[-1000:])))
+    assert (got.requests, got.scheduled_requests, got.cache_size_in_bytes) == (5, 3, 1 << 20)
+    waited = []
+    with t.time_forward(lambda: waited.append(1)):
+        pass
+    assert waited == [1] and 0.0 < t.get_metrics().inference_duration < 1e6
+    t.reset_cache_usage_statistics()            # :791-795: maximum and average start over, the last usage stays
+    got = t.get_metrics()
+    assert (got.max_cache_usage, got.avg_cache_usage) == (0.0, 0.0) and got.cache_usage == usages[-1]
+    t.register_step([8], 16)
+    assert t.get_metrics().avg_cache_usage == 50.0
+
+
 def test_xattention_threshold_schedule(pkg):
     """Scheduler::_schedule_xattention_threshold (scheduler.hpp:922-940): library against the checker's restatement."""
     from oracle import oracle as O

@@ -29,7 +29,9 @@ NUM_LAYERS_FOR_TOKS = 32  # Llama-3-8B depth: tok/s = batch / (32 * t_layer), at
 # (a workload without a reading of the kernel as it stands is not listed: `traffic` is then null)
 MEASURED_TRAFFIC = {
     "llama3_8b_decode_u8_b64_ctx4096": (585.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
-    "qwen25_7b_mixed_bf16": (835.0e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
+    "llama3_8b_eviction_u8_b256_ctx8192": (4656.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_eviction_u8_b256_ctx8192.md"),
+    "long_context_decode_u8_b8_ctx32768": (594.4e6, "profiles/pa_decode_u8_kernel__long_context_decode_u8_b8_ctx32768.md"),
+    "qwen25_7b_mixed_bf16": (843.1e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
 }
 
 
@@ -55,7 +57,7 @@ def parse():
                     help="decoder layers of the eviction leg of --config 4 (score registration and eviction run over "
                          "every layer of every sequence in one call)")
     ap.add_argument("--evict-modes", default="norm_sum,kvcrush,adaptive_rkv",
-                    help="eviction legs of --config 4 beside NORM_SUM: kvcrush, adaptive_rkv (comma separated)")
+                    help="eviction legs of --config 4 beside NORM_SUM: kvcrush, adaptive_rkv (comma separated); none = no eviction leg")
     ap.add_argument("--diversity", type=int, default=0, metavar="TOKENS",
                     help="adds a leg: ADAPTIVE_RKV block diversity over an evictable area of this many tokens (a "
                          "multiple of 32) of every sequence, behind a start area of 32 tokens")
@@ -625,7 +627,7 @@ def main():
         res["cache_rotation"] = rotation_leg(torch, pkg, op, spec, kc, dev)
     if args.kv_cache_leg:
         res["kv_cache"] = kv_cache_leg(torch, pkg, dev)
-    if args.config == 4:
+    if args.config == 4 and args.evict_modes != "none":
         res["eviction"] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers)
         for mode in [m for m in args.evict_modes.split(",") if m and m != "norm_sum"]:
             res["eviction_" + mode] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers, mode)

@@ -749,7 +749,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
                    PA_NOT_IMPLEMENTED,
                    "pa_attention_static serves steps in which every sequence schedules one token, over a u8 cache or a "
-                   "16-bit cache of the query's type (block size 32 or 16, head size 64 or 128, at most 16 heads per kv head)");
+                   "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64 or 128, K and V alike; at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
     if (use_decode) {

@@ -22,8 +22,12 @@ def _run(torch, op, case, dev, static, want_scores=True):
     op.set_block_indices(case["block_indices"], case["num_blocks"])
     out = torch.full_like(q, float("nan"))
     scores = torch.full((op.total_scores,), float("nan"), dtype=torch.float32, device=dev) if want_scores else None
+    torch.cuda.synchronize(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]
     (op.attention_static if static else op.attention)(q, kc, vc, out, scores)
     op.synchronize()
+    if static:  # nothing was allocated (or freed) on the device inside the call
+        assert torch.cuda.mem_get_info(dev)[0] == free_before
     torch.cuda.synchronize(dev)
     return (out.view(torch.int16).cpu().numpy().view(np.uint16), scores.cpu().numpy() if want_scores else None,
             op.num_splits)

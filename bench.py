@@ -577,7 +577,10 @@ def main():
     mixed = T > B  # multi-token sequences present: the MFMA kernel is the dominant one
     traffic, traffic_source = MEASURED_TRAFFIC.get(spec["name"], (None, None)) \
         if with_scores and args.batch is None and not args.kv_dtype else (None, None)
-    flops = wl.attention_flops(spec)
+    # the matrix kernel is priced with the flops of the multi-token sequences only: the single-token sequences of a
+    # mixed step run in a decode kernel (over 16-bit caches next to it on a second stream, so its launch time includes
+    # what it loses to the neighbour)
+    flops = wl.attention_flops(spec, multi_token_only=mixed)
     res = {
         "metric": "paged-attn decode GB/s (tok/s and % HBM peak alongside), Llama-3-8B shape, u8 KV, 1 GPU"
                   if args.config == 2 and spec["kv_dtype"] == "u8" else

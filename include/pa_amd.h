@@ -73,7 +73,10 @@ typedef struct pa_config {
                                 (src/cpp/src/utils.cpp:840-863); the key cache's type, and the value cache's unless
                                 value_cache_dtype_p1 says otherwise */
     int32_t num_layers;      /* decoder layers (block tables may differ per layer with eviction) */
-    void* stream;            /* hipStream_t to launch on; NULL = the device's default stream */
+    void* stream;            /* hipStream_t to launch on; NULL = the device's default stream.  Everything a call
+                                queues is ordered with this stream: in a mixed step over a 16-bit cache one of its
+                                two kernels runs on a second stream of the context's own, forked from this stream
+                                and joined back into it by events inside the call */
     /* The value side where it differs from the key side: a model's value_cache.<L> may have another head size and
      * another precision than its key_cache.<L> (the reference keeps shape and precision per tensor,
      * src/cpp/src/continuous_batching/cache/kv_cache_manager.hpp:74-92, and reads the V head size on its own,

@@ -2,7 +2,6 @@
 // C++ behind `extern "C"`; no exception leaves this file.
 #include <algorithm>
 #include <cmath>
-#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <stdexcept>
@@ -202,6 +201,11 @@ struct pa_ctx {
     // optional per-kernel timing
     bool profiling = false, timed = false;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // A mixed step over a 16-bit cache: the single-token sequences' decode kernel runs on a second stream next to the
+    // matrix kernel of the chunks (forked and joined with events, so the caller only ever sees the context's stream).
+    hipStream_t side = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    bool split16 = false;  // this step: single-token items are listed behind the chunk items and left to the decode kernel
 };
 
 // Every tensor (K and V of every layer) is a reserved range of virtual addresses whose front is backed by physical
@@ -525,6 +529,20 @@ void plan_items(pa_ctx* ctx) {
     const bool split_off_decode = decode_u8_shape(ctx->cfg);
     ctx->h_dec.clear();
     ctx->h_dec16.clear();
+    // A mixed step over a 16-bit cache with the 16-bit decode kernel available: chunk items and single-token
+    // sequences do not share a launch -- the chunks go to the straight-to-LDS variant, the single-token sequences to
+    // the decode kernel on a second stream, side by side.  Their items are still listed (behind the chunks' items, where
+    // the matrix kernel passes them over) but count for nothing in the plan of the chunks.
+    {
+        bool any_single = false, any_chunk = false;
+        for (int32_t b = 0; b < B; ++b) {
+            const int32_t q_len = sb[b + 1] - sb[b];
+            any_single = any_single || q_len == 1;
+            any_chunk = any_chunk || (q_len > 1 && xatt_seq_index(ctx, b) < 0);
+        }
+        ctx->split16 = narrow_all && any_single && any_chunk && decode16_shape(ctx->cfg) && ctx->cfg.head_size == 128;
+    }
+    size_t planned_tiles = 0;
     for (int32_t b = 0; b < B; ++b) {
         const int32_t q_len = sb[b + 1] - sb[b];
         if (split_off_decode && q_len == 1) {
@@ -540,22 +558,25 @@ void plan_items(pa_ctx* ctx) {
             const int32_t last_pos = past[b] + q0 + nq - 1;
             const int32_t first_pos = sw > 0 ? std::max(0, past[b] + q0 + 1 - sw) : 0;
             tiles.push_back({b, q0, nq, first_pos / 32, last_pos / 32 + 1, sparse ? 3 : q_len == 1 ? 2 : (nq * G > 16 ? 0 : 1)});
+            if (q_len == 1 && ctx->split16) continue;  // (another kernel's work)
             total_blocks += last_pos / 32 + 1 - first_pos / 32;
+            ++planned_tiles;
         }
     }
     // Ranges of at least 8 blocks -- of at least 16 once the uncut tiles alone make three quarters of a round of
     // workgroups: cutting their short items further adds workgroups nobody waits for and a merge pass for their rows
     // (four 512-token prompts from scratch: 42.8 -> 33.6 us over bf16, 56.5 -> 44.4 us over u8; a single one, whose 116
     // to 128 workgroups leave most of the chip idle, is better off cut: 29.9 against 35.2 us over u8).
-    const bool round_filled = (int64_t)tiles.size() * ctx->cfg.num_kv_heads >= 384;
+    const bool round_filled = (int64_t)planned_tiles * ctx->cfg.num_kv_heads >= 384;
     const int64_t shortest = round_filled ? 16 : 8;
     int64_t target = std::min<int64_t>(128, std::max<int64_t>(shortest, total_blocks * ctx->cfg.num_kv_heads / 768));
     // ... and tiles of about one length that fill the round by themselves are not cut at all: there is nothing to
     // balance (32 sequences x 64 tokens behind 500: 62.6 -> 42.6 us over bf16, 77.2 -> 56.1 us over u8)
     if (round_filled && !tiles.empty()) {
         int64_t longest = 0;
-        for (const Tile& t : tiles) longest = std::max<int64_t>(longest, t.hi - t.lo);
-        if (2 * longest * (int64_t)tiles.size() <= 3 * total_blocks) target = std::min<int64_t>(128, std::max(target, longest));
+        for (const Tile& t : tiles)
+            if (!(t.kind == 2 && ctx->split16)) longest = std::max<int64_t>(longest, t.hi - t.lo);
+        if (2 * longest * (int64_t)planned_tiles <= 3 * total_blocks) target = std::min<int64_t>(128, std::max(target, longest));
     }
     // single-token sequences as items of the kernel variant that can hand their probabilities to the score kernel
     const bool stash_ok = narrow_all && G <= 16;
@@ -612,7 +633,7 @@ void plan_items(pa_ctx* ctx) {
         // (the single-token items longest first as well: 0.272 -> 0.266 ms on the same workload)
         std::stable_sort(items.begin() + n_multi, items.begin() + n_multi + n_s,
                          [](const pa::PrefillItem& x, const pa::PrefillItem& y) { return x.te - x.tb > y.te - y.tb; });
-        if (narrow_all && n_s > 0 && n_multi > 0 && cost_s > 0.3 * cost_m) {
+        if (narrow_all && n_s > 0 && n_multi > 0 && cost_s > 0.3 * cost_m && !ctx->split16) {
             std::vector<pa::PrefillItem> mixed;
             mixed.reserve(items.size());
             int32_t im = 0, is = 0;
@@ -742,8 +763,9 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     // 16-bit caches, no dense chunk in the step: the single-token sequences go to their own decode kernel.  (Next to
     // dense chunks they stay work items of the matrix kernel: bandwidth-bound and matrix-bound items share the CUs
     // inside one launch, which two launches one after the other do not.)
+    const bool side_by_side = ctx->split16 && !static_ws;
     const bool use_decode16 = use_mfma && decode16_shape(c) && !ctx->h_dec16.empty() &&
-                              ctx->n_single + ctx->n_sparse == ctx->n_items;
+                              (ctx->n_single + ctx->n_sparse == ctx->n_items || side_by_side);
     const bool mfma_left = use_mfma && !(use_decode16 && ctx->n_single == ctx->n_items);
     if (static_ws)
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
@@ -811,8 +833,20 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.final_ml = ws.final_ml;
         a.group_scores = ws.group_scores;
         a.p_split = ws.p_split;
-        HIP_CHECK(pa::launch_decode16(ctx->stream, a, c.query_dtype, io->scores, ctx->max_kv, mfma_left ? nullptr : ev0,
+        hipStream_t s16 = ctx->stream;
+        if (side_by_side) {  // fork: the decode kernel starts behind what the context's stream holds so far
+            if (!ctx->side) {
+                HIP_CHECK(hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking));
+                HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+                HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+            }
+            HIP_CHECK(hipEventRecord(ctx->ev_fork, ctx->stream));
+            HIP_CHECK(hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0));
+            s16 = ctx->side;
+        }
+        HIP_CHECK(pa::launch_decode16(s16, a, c.query_dtype, io->scores, ctx->max_kv, mfma_left ? nullptr : ev0,
                                       mfma_left ? nullptr : ev1));
+        if (side_by_side) HIP_CHECK(hipEventRecord(ctx->ev_join, ctx->side));
         ctx->timed = ctx->profiling;
     }
     if (mfma_left) {
@@ -912,6 +946,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                                                a.xatt, ss, mg));
         }
     }
+    if (use_decode16 && side_by_side) HIP_CHECK(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));  // join
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;
     ctx->part_acc.reserve(rows * ctx->nsplit * v_head(c) * sizeof(float));
@@ -981,6 +1016,9 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->x_sums.release();
     ctx->x_mask.release();
     ctx->x_item_keep.release();
+    if (ctx->side) (void)hipStreamDestroy(ctx->side);
+    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;

@@ -79,12 +79,15 @@ def algorithmic_bytes(spec, with_scores=True):
     return dict(kv=kv_bytes, q_out=q_out, ints=ints, scores=scores, total=kv_bytes + q_out + ints + scores)
 
 
-def attention_flops(spec):
-    """Matrix flops of one attention call: 4 * D per (query row, visible position), all query heads."""
+def attention_flops(spec, multi_token_only=False):
+    """Matrix flops of one attention call: 4 * D per (query row, visible position), all query heads
+    (multi_token_only: of the sequences that schedule more than one token)."""
     past = spec["past_lens"].astype(np.int64)
     new = np.diff(spec["subsequence_begins"]).astype(np.int64)
     pairs = 0
     for p, n in zip(past, new):
+        if multi_token_only and n <= 1:
+            continue
         last = p + np.arange(n, dtype=np.int64)  # last visible position of each new token
         vis = last + 1
         if spec["sliding_window"] > 0:

@@ -774,6 +774,22 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                    "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64 or 128, K and V alike; at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
+    // fork: what is launched on the returned stream starts behind what the context's stream holds so far and runs
+    // next to what follows on it, until the join at the end of this call
+    bool forked = false;
+    auto fork_side = [&]() -> hipStream_t {
+        if (!ctx->side) {
+            HIP_CHECK(hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking));
+            HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+            HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+        }
+        if (!forked) {
+            HIP_CHECK(hipEventRecord(ctx->ev_fork, ctx->stream));
+            HIP_CHECK(hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0));
+            forked = true;
+        }
+        return ctx->side;
+    };
     if (use_decode) {
         pa::DecodeArgs a{};
         a.st = ctx->dev;
@@ -803,8 +819,9 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.final_ml = ws.final_ml;
         a.group_scores = ws.group_scores;
         a.p_split = ws.p_split;
-        HIP_CHECK(pa::launch_decode_u8(ctx->stream, a, c.query_dtype, io->scores, ctx->max_kv,
-                                       use_mfma ? nullptr : ev0, use_mfma ? nullptr : ev1));
+        // (next to the matrix kernel of a mixed step: on the second stream, like the 16-bit decode kernel below)
+        HIP_CHECK(pa::launch_decode_u8(use_mfma && !static_ws ? fork_side() : ctx->stream, a, c.query_dtype, io->scores,
+                                       ctx->max_kv, use_mfma ? nullptr : ev0, use_mfma ? nullptr : ev1));
         ctx->timed = ctx->profiling;
     }
     if (use_decode16) {
@@ -833,20 +850,8 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         a.final_ml = ws.final_ml;
         a.group_scores = ws.group_scores;
         a.p_split = ws.p_split;
-        hipStream_t s16 = ctx->stream;
-        if (side_by_side) {  // fork: the decode kernel starts behind what the context's stream holds so far
-            if (!ctx->side) {
-                HIP_CHECK(hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking));
-                HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
-                HIP_CHECK(hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
-            }
-            HIP_CHECK(hipEventRecord(ctx->ev_fork, ctx->stream));
-            HIP_CHECK(hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0));
-            s16 = ctx->side;
-        }
-        HIP_CHECK(pa::launch_decode16(s16, a, c.query_dtype, io->scores, ctx->max_kv, mfma_left ? nullptr : ev0,
-                                      mfma_left ? nullptr : ev1));
-        if (side_by_side) HIP_CHECK(hipEventRecord(ctx->ev_join, ctx->side));
+        HIP_CHECK(pa::launch_decode16(side_by_side ? fork_side() : ctx->stream, a, c.query_dtype, io->scores, ctx->max_kv,
+                                      mfma_left ? nullptr : ev0, mfma_left ? nullptr : ev1));
         ctx->timed = ctx->profiling;
     }
     if (mfma_left) {
@@ -946,7 +951,10 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
                                                a.xatt, ss, mg));
         }
     }
-    if (use_decode16 && side_by_side) HIP_CHECK(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));  // join
+    if (forked) {  // join
+        HIP_CHECK(hipEventRecord(ctx->ev_join, ctx->side));
+        HIP_CHECK(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));
+    }
     if (use_decode || use_mfma) return;  // (use_decode16 implies use_mfma)
     ctx->nsplit = ctx->generic_nsplit;
     ctx->part_acc.reserve(rows * ctx->nsplit * v_head(c) * sizeof(float));

@@ -13,45 +13,13 @@
 namespace pa {
 namespace {
 
-// A row per 16 lanes, each lane D / 16 consecutive elements (16-byte loads at D = 128), four rows per wave.  A wave
-// takes four consecutive tokens of one kv head, so that what it writes is one run of cache bytes wherever the
-// tokens share a block.  Minimum and maximum of a row are reduced over its 16 lanes with four
-// cross-lane (DPP) steps; the arithmetic per element is that of quantize_row_u8, so the bytes are the same.
-template <int QDT, int KVDT, int E>
-__global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ key,
-                                                        const uint16_t* __restrict__ value,
-                                                        uint8_t* __restrict__ key_cache,
-                                                        uint8_t* __restrict__ value_cache,
-                                                        const int32_t* __restrict__ block_indices) {
-#pragma clang fp contract(off)
-    static_assert(E == 4 || E == 8, "D = 64 or 128");
-    constexpr int D = 16 * E;
-    const int l16 = threadIdx.x & 15;
-    const long per_tensor = (long)st.T * sh.Hkv;
-    long row = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;  // (K | V, kv head, token)
-    // (rows beyond the end repeat the last one: no divergence around the cross-lane steps, and the same bytes twice)
-    row = min(row, 2 * per_tensor - 1);
-    const int which = row >= per_tensor;
-    const long rem = row - which * per_tensor;
-    const int h = (int)(rem / st.T), t = (int)(rem % st.T);
-    const int b = st.token_seq[t];
-    const int slot = st.past_lens[b] + (t - st.subsequence_begins[b]);
-    const long phys = block_indices[st.block_indices_begins[b] + slot / sh.bs];
-    constexpr int RB = KVDT == DT_U8 ? D + 8 : 2 * D;
-    const uint16_t* src = (which ? value : key) + ((long)t * sh.Hkv + h) * D + l16 * E;
-    uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)RB;
+constexpr int TOKENS_KERNEL_MIN_T = 8192;  // steps of this many tokens take the kernel that walks a token's rows
 
-    uint32_t w[E / 2];
-    if constexpr (E == 4) {
-        const uint2 v = *reinterpret_cast<const uint2*>(src);
-        w[0] = v.x; w[1] = v.y;
-    } else {
-#pragma unroll
-        for (int i = 0; i < E / 8; ++i) {
-            const uint4 v = *reinterpret_cast<const uint4*>(src + 8 * i);
-            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
-        }
-    }
+// One row's 16 lanes: `w` holds the lane's E elements as loaded, `dst` is the row in the cache.
+template <int QDT, int KVDT, int E>
+__device__ __forceinline__ void append_row(uint32_t (&w)[E / 2], uint8_t* dst, int l16) {
+#pragma clang fp contract(off)
+    constexpr int D = 16 * E;
     if constexpr (KVDT == DT_U8) {
         float x[E];
 #pragma unroll
@@ -95,6 +63,95 @@ __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, co
     }
 }
 
+template <int E>
+__device__ __forceinline__ void load_row(uint32_t (&w)[E / 2], const uint16_t* src) {
+    if constexpr (E == 4) {
+        const uint2 v = *reinterpret_cast<const uint2*>(src);
+        w[0] = v.x; w[1] = v.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < E / 8; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(src + 8 * i);
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+        }
+    }
+}
+
+// A row per 16 lanes, each lane D / 16 consecutive elements (16-byte loads at D = 128), four rows per wave.  A wave
+// takes four consecutive tokens of one kv head, so that what it writes is one run of cache bytes wherever the
+// tokens share a block.  Minimum and maximum of a row are reduced over its 16 lanes with four
+// cross-lane (DPP) steps; the arithmetic per element is that of quantize_row_u8, so the bytes are the same.
+template <int QDT, int KVDT, int E>
+__global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ key,
+                                                        const uint16_t* __restrict__ value,
+                                                        uint8_t* __restrict__ key_cache,
+                                                        uint8_t* __restrict__ value_cache,
+                                                        const int32_t* __restrict__ block_indices) {
+#pragma clang fp contract(off)
+    static_assert(E == 4 || E == 8, "D = 64 or 128");
+    constexpr int D = 16 * E;
+    const int l16 = threadIdx.x & 15;
+    const long per_tensor = (long)st.T * sh.Hkv;
+    long row = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;  // (K | V, kv head, token)
+    // (rows beyond the end repeat the last one: no divergence around the cross-lane steps, and the same bytes twice)
+    row = min(row, 2 * per_tensor - 1);
+    const int which = row >= per_tensor;
+    const long rem = row - which * per_tensor;
+    const int h = (int)(rem / st.T), t = (int)(rem % st.T);
+    const int b = st.token_seq[t];
+    const int slot = st.past_lens[b] + (t - st.subsequence_begins[b]);
+    const long phys = block_indices[st.block_indices_begins[b] + slot / sh.bs];
+    constexpr int RB = KVDT == DT_U8 ? D + 8 : 2 * D;
+    const uint16_t* src = (which ? value : key) + ((long)t * sh.Hkv + h) * D + l16 * E;
+    uint8_t* dst = (which ? value_cache : key_cache) + ((phys * sh.Hkv + h) * sh.bs + slot % sh.bs) * (long)RB;
+
+    uint32_t w[E / 2];
+    load_row<E>(w, src);
+    append_row<QDT, KVDT, E>(w, dst, l16);
+}
+
+// Steps of many tokens (a prompt's chunk): sixteen lanes own one TOKEN and walk its 2 * Hkv rows (K then V, kv heads
+// in order), four rows' loads in flight.  The chain of dependent loads that leads to a row's place in the cache
+// (token -> sequence -> position -> block id) is walked once per token instead of once per row, and a lane has four
+// times the bytes in flight: with a row per 16 lanes that chain, not the memory system, set the pace (3.2 TB/s into a
+// u8 cache at 131072 tokens x 8 kv heads).
+template <int QDT, int KVDT, int E>
+__global__ __launch_bounds__(256) void kv_append_tokens_kernel(StepDev st, Shape sh, const uint16_t* __restrict__ key,
+                                                               const uint16_t* __restrict__ value,
+                                                               uint8_t* __restrict__ key_cache,
+                                                               uint8_t* __restrict__ value_cache,
+                                                               const int32_t* __restrict__ block_indices) {
+    static_assert(E == 4 || E == 8, "D = 64 or 128");
+    constexpr int D = 16 * E, U = 4;
+    constexpr int RB = KVDT == DT_U8 ? D + 8 : 2 * D;
+    const int l16 = threadIdx.x & 15;
+    // (tokens beyond the end repeat the last one: no divergence around the cross-lane steps, and the same bytes twice)
+    const int t = min((int)blockIdx.x * 16 + (int)(threadIdx.x >> 4), st.T - 1);
+    const int b = st.token_seq[t];
+    const int slot = st.past_lens[b] + (t - st.subsequence_begins[b]);
+    const long phys = block_indices[st.block_indices_begins[b] + slot / sh.bs];
+    const long dst_tok = (phys * sh.Hkv * sh.bs + slot % sh.bs) * (long)RB;  // the token's row of kv head 0
+    const long head_stride = (long)sh.bs * RB;
+    const uint16_t* src_tok = nullptr;
+    const int rows = 2 * sh.Hkv;
+    for (int j0 = 0; j0 < rows; j0 += U) {
+        uint32_t w[U][E / 2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = min(j0 + u, rows - 1);  // (a last group that is not full repeats the last row)
+            const int which = j >= sh.Hkv, h = j - which * sh.Hkv;
+            src_tok = (which ? value : key) + ((long)t * sh.Hkv + h) * D + l16 * E;
+            load_row<E>(w[u], src_tok);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = min(j0 + u, rows - 1);
+            const int which = j >= sh.Hkv, h = j - which * sh.Hkv;
+            append_row<QDT, KVDT, E>(w[u], (which ? value_cache : key_cache) + dst_tok + h * head_stride, l16);
+        }
+    }
+}
+
 template <int QDT, int KVDT>
 hipError_t launch_epl(hipStream_t s, const StepDev& st, const Shape& sh, const void* key, const void* value,
                       void* kc, void* vc, const int32_t* bi) {
@@ -105,6 +162,15 @@ hipError_t launch_epl(hipStream_t s, const StepDev& st, const Shape& sh, const v
     auto v = reinterpret_cast<const uint16_t*>(value);
     auto kcu = reinterpret_cast<uint8_t*>(kc);
     auto vcu = reinterpret_cast<uint8_t*>(vc);
+    if (st.T >= TOKENS_KERNEL_MIN_T) {  // enough tokens to fill the chip with a token per 16 lanes
+        const dim3 tgrid((unsigned)((st.T + 15) / 16));
+        switch (sh.D / 64) {
+            case 1: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 4>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+            case 2: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 8>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+            default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     switch (sh.D / 64) {
         case 1: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 4>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
         case 2: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 8>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;

@@ -80,14 +80,30 @@ MANY_ROWS = [
 
 @pytest.mark.parametrize("qd,kd,D,Hkv,bs", MANY_ROWS)
 def test_kv_append_many_rows_bit_exact(pkg, dev, qd, kd, D, Hkv, bs):
+    T_min = 16384 // (2 * Hkv) + 70
+    _append_many(pkg, dev, qd, kd, D, Hkv, bs, [T_min - 700, 333, 1, 300, 65, 1], 16384)
+
+
+MANY_TOKENS = [
+    # steps of 8192 or more tokens take the append kernel in which 16 lanes own a token and walk its rows four at a
+    # time (3 kv heads: the last group of rows is not full)
+    ("f16", "u8", 128, 8, 32), ("bf16", "u8", 64, 3, 32), ("f16", "u8", 128, 1, 16), ("bf16", "bf16", 128, 4, 32),
+    ("f16", "bf16", 64, 3, 64), ("bf16", "f16", 128, 2, 32),
+]
+
+
+@pytest.mark.parametrize("qd,kd,D,Hkv,bs", MANY_TOKENS)
+def test_kv_append_many_tokens_bit_exact(pkg, dev, qd, kd, D, Hkv, bs):
+    _append_many(pkg, dev, qd, kd, D, Hkv, bs, [7000, 333, 1, 1300, 65, 1], 8192 * Hkv * 2)
+
+
+def _append_many(pkg, dev, qd, kd, D, Hkv, bs, new, min_rows):
     import torch
     from oracle import oracle as O
-    T_min = 16384 // (2 * Hkv) + 70
-    new = [T_min - 700, 333, 1, 300, 65, 1]
     case = H.case_from_lens(f"append_many_{qd}_{kd}_{D}", Hkv, Hkv, D, bs, qd, kd, [0, 31, 4000, 100, 7, 0], new)
     print(f"case {case['name']} seed 9", flush=True)
     c = H.build_case(case, 9, outliers=True)
-    assert int(c["subsequence_begins"][-1]) * Hkv * 2 >= 16384
+    assert int(c["subsequence_begins"][-1]) * Hkv * 2 >= min_rows
     # rows with a zero range, a huge range and exact ties, in the middle of the long sequence
     x = np.zeros((3, Hkv * D), np.float32)
     x[0] = 3.25

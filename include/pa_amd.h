@@ -143,8 +143,7 @@ typedef struct pa_layer_io {
     float* scores;
 } pa_layer_io;
 
-/* One layer's PagedAttention: KV append (+ u8 / u4 quantisation), attention, optional scores.  The op's `alibi_slopes`
- * input has no counterpart: no ALiBi term is applied, and a binding must refuse a non-empty slopes tensor.  Tuned
+/* One layer's PagedAttention: KV append (+ u8 / u4 quantisation), attention, optional scores.  Tuned
  * kernels serve block_size 16, 32, 64, 128 and 256 with head size 64 or 128, K and V alike, over a u8 cache or an f16 /
  * bf16 cache of the query's type; every other combination pa_create accepts (other head sizes, a value head size or
  * value precision of its own, u4 rows, a 16-bit cache of the other 16-bit type, other block sizes) runs on shape-generic
@@ -152,6 +151,15 @@ typedef struct pa_layer_io {
  * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
  * writes). */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
+/* The op's `alibi_slopes` input (input 11: f32 [num_heads]; a graph constant that SDPAToPagedAttention leaves empty
+ * for models without ALiBi, and that the reference never sets itself): with slopes set, every logit gets
+ * slope[head] * (key position - query position) added after the scaling.  `slopes` is a host array of `count` =
+ * num_heads values; count 0 (or all zeros) takes the term away again.  A model constant: set it once after pa_create
+ * (a step that has begun must begin again after a change).  The tuned kernels have no such term: a context with
+ * slopes runs on the shape-generic kernels, block-sparse prefill is refused.  Parity with the plugin's term is
+ * unpinned (it is applied inside the op; this is the formula of the ALiBi paper). */
+int32_t pa_set_alibi_slopes(pa_ctx* ctx, const float* slopes, int32_t count);
+
 /* The two halves of pa_forward on their own (same arguments; pa_kv_append ignores query/out/scores,
  * pa_attention ignores key/value). */
 int32_t pa_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);

@@ -22,7 +22,7 @@ STATUS_NAMES = {0: "OK", -1: "GENERAL_ERROR", -2: "NOT_IMPLEMENTED", -4: "PARAME
 # every symbol include/pa_amd.h declares
 EXPORTS = [
     "pa_version", "pa_global_last_error", "pa_create", "pa_destroy", "pa_last_error", "pa_step_begin",
-    "pa_set_block_indices", "pa_set_block_indices_layers", "pa_forward", "pa_kv_append", "pa_attention", "pa_attention_static", "pa_synchronize", "pa_get_num_splits", "pa_set_profiling", "pa_last_kernel_ms",
+    "pa_set_block_indices", "pa_set_block_indices_layers", "pa_set_alibi_slopes", "pa_forward", "pa_kv_append", "pa_attention", "pa_attention_static", "pa_synchronize", "pa_get_num_splits", "pa_set_profiling", "pa_last_kernel_ms",
     "pa_pack_step", "pa_snapkv_num_scores", "pa_kv_cache_create", "pa_kv_cache_create_layers", "pa_kv_cache_destroy", "pa_kv_cache_last_error",
     "pa_kv_cache_block_bytes", "pa_kv_cache_allocate", "pa_kv_cache_num_blocks", "pa_kv_cache_get",
     "pa_kv_cache_copy_blocks", "pa_normalize_num_kv_blocks", "pa_evictor_create", "pa_score_manager_create",
@@ -106,6 +106,7 @@ def lib():
         "pa_step_begin": (i32, [vp, P(pa_step_meta)]),
         "pa_set_block_indices": (i32, [vp, i32, P(i32), i32, i64]),
         "pa_set_block_indices_layers": (i32, [vp, i32, i32, P(P(i32)), i32, i64]),
+        "pa_set_alibi_slopes": (i32, [vp, P(C.c_float), i32]),
         "pa_forward": (i32, [vp, i32, P(pa_layer_io)]),
         "pa_kv_append": (i32, [vp, i32, P(pa_layer_io)]),
         "pa_attention": (i32, [vp, i32, P(pa_layer_io)]),

@@ -176,6 +176,7 @@ struct AttnWorkspace {
     float* logits;     // [Hq, total_scores] raw scaled logits of single-token sequences (scores only)
     int32_t nsplit;
     int32_t total_scores;
+    const float* alibi = nullptr;  // [Hq] ALiBi slopes, or null: logit += slope * (key position - query position)
 };
 
 // What the shape-generic kernels take: a head size and an element type per cache tensor (query and key rows have Dk

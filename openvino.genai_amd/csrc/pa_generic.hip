@@ -112,6 +112,7 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, GenericShap
     const int32_t* table = block_indices + st.block_indices_begins[b];
     const bool keep_logits = store_logits && q_len == 1 && st.score_window[b] > 0;
     float* logit_row = ws.logits + (long)hq * ws.total_scores + st.score_offsets[b];
+    const float slope = ws.alibi ? ws.alibi[hq] : 0.0f;
 
     float m = -INFINITY, l = 0.0f;
     float acc[EPL];
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, GenericShap
 #pragma unroll
                 for (int e = 0; e < 8; ++e) dot += qs[wv][d + e] * k8[e];
             }
-            s = dot;
+            s = ws.alibi ? dot + slope * (float)(j - last) : dot;
             if (keep_logits) logit_row[j] = s;
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -257,6 +258,7 @@ __global__ __launch_bounds__(256) void pa_scores_window_kernel(StepDev st, Gener
                         dot += load16<QDT>((uint16_t)(w[e] >> 16)) * st.scale * k8[2 * e + 1];
                     }
                 }
+                if (ws.alibi) dot += ws.alibi[h] * (float)(j - last);
                 const float M = ws.final_ml[2 * ((long)(t0 + i) * sh.Hq + h)];
                 const float L = ws.final_ml[2 * ((long)(t0 + i) * sh.Hq + h) + 1];
                 sum += __expf(dot - M) / L;

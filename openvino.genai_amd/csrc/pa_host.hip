@@ -205,7 +205,11 @@ struct pa_ctx {
     // matrix kernel of the chunks (forked and joined with events, so the caller only ever sees the context's stream).
     hipStream_t side = nullptr;
     hipEvent_t ev_fork = nullptr, ev_join = nullptr;
-    bool split16 = false;  // this step: single-token items are listed behind the chunk items and left to the decode kernel
+    bool split16 = false;
+    // ALiBi (the op's alibi_slopes input): a slope per query head on the device; the tuned kernels have no such term,
+    // so a context with slopes runs on the shape-generic kernels
+    DevBuf alibi;
+    bool has_alibi = false;  // this step: single-token items are listed behind the chunk items and left to the decode kernel
 };
 
 // Every tensor (K and V of every layer) is a reserved range of virtual addresses whose front is backed by physical
@@ -359,6 +363,11 @@ bool decode16_shape(const pa_config& c) {
     return kv_alike(c) && c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && tuned_block_size(c.block_size) &&
            (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
 }
+
+// The same questions asked of a context: one with ALiBi slopes has no tuned attention kernel.
+bool decode_u8_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode_u8_shape(ctx->cfg); }
+bool mfma_shape(const pa_ctx* ctx) { return !ctx->has_alibi && mfma_shape(ctx->cfg); }
+bool decode16_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode16_shape(ctx->cfg); }
 
 // Split-K plan of the decode kernels: workgroups per (sequence, kv head) and the most blocks one walks.
 void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, int32_t* max_tiles_out,
@@ -526,7 +535,7 @@ void plan_items(pa_ctx* ctx) {
     int32_t n_single_seqs = 0;
     std::vector<Tile> tiles;
     int64_t total_blocks = 0;
-    const bool split_off_decode = decode_u8_shape(ctx->cfg);
+    const bool split_off_decode = decode_u8_shape(ctx);
     ctx->h_dec.clear();
     ctx->h_dec16.clear();
     // A mixed step over a 16-bit cache with the 16-bit decode kernel available: chunk items and single-token
@@ -540,7 +549,7 @@ void plan_items(pa_ctx* ctx) {
             any_single = any_single || q_len == 1;
             any_chunk = any_chunk || (q_len > 1 && xatt_seq_index(ctx, b) < 0);
         }
-        ctx->split16 = narrow_all && any_single && any_chunk && decode16_shape(ctx->cfg) && ctx->cfg.head_size == 128;
+        ctx->split16 = narrow_all && any_single && any_chunk && decode16_shape(ctx) && ctx->cfg.head_size == 128;
     }
     size_t planned_tiles = 0;
     for (int32_t b = 0; b < B; ++b) {
@@ -758,13 +767,13 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     const int32_t* table = table_for(ctx, layer);
     const pa_config& c = ctx->cfg;
     const size_t rows = (size_t)ctx->T * c.num_heads;
-    const bool use_decode = decode_u8_shape(c) && !ctx->h_dec.empty();
-    const bool use_mfma = mfma_shape(c) && ctx->n_items > 0;
+    const bool use_decode = decode_u8_shape(ctx) && !ctx->h_dec.empty();
+    const bool use_mfma = mfma_shape(ctx) && ctx->n_items > 0;
     // 16-bit caches, no dense chunk in the step: the single-token sequences go to their own decode kernel.  (Next to
     // dense chunks they stay work items of the matrix kernel: bandwidth-bound and matrix-bound items share the CUs
     // inside one launch, which two launches one after the other do not.)
     const bool side_by_side = ctx->split16 && !static_ws;
-    const bool use_decode16 = use_mfma && decode16_shape(c) && !ctx->h_dec16.empty() &&
+    const bool use_decode16 = use_mfma && decode16_shape(ctx) && !ctx->h_dec16.empty() &&
                               (ctx->n_single + ctx->n_sparse == ctx->n_items || side_by_side);
     const bool mfma_left = use_mfma && !(use_decode16 && ctx->n_single == ctx->n_items);
     if (static_ws)
@@ -937,7 +946,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
             ss.n_seqs = (int32_t)ctx->h_dec16.size();
         }
         // (without the single-token sequences the launch has rows for the listed multi-token sequences only)
-        const bool singles_too = !(decode_u8_shape(c) || use_decode16 || hand_over);
+        const bool singles_too = !(decode_u8_shape(ctx) || use_decode16 || hand_over);
         const int32_t replay_seqs = singles_too ? ctx->B : (int32_t)ctx->h_multi.size();
         const bool merge_later = score_launch && a.n_merge > 0 && replay_seqs + ss.n_seqs > 0 && ctx->max_kv > 0;
         HIP_CHECK(pa::launch_prefill16(ctx->stream, a, c.query_dtype, c.kv_cache_dtype, ev0, ev1, merge_later));
@@ -962,7 +971,8 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     ctx->final_ml.reserve(rows * 2 * sizeof(float));
     if (io->scores) ctx->logits.reserve((size_t)c.num_heads * ctx->total_scores * sizeof(float));
     pa::AttnWorkspace ws{ctx->part_acc.as<float>(), ctx->part_ml.as<float>(), ctx->final_ml.as<float>(),
-                         ctx->logits.as<float>(), ctx->nsplit, ctx->total_scores};
+                         ctx->logits.as<float>(), ctx->nsplit, ctx->total_scores,
+                         ctx->has_alibi ? ctx->alibi.as<float>() : nullptr};
     HIP_CHECK(pa::launch_attention_generic(ctx->stream, ctx->dev, generic_shape_of(c), c.query_dtype,
                                            io->query, io->key_cache, io->value_cache, table, ws, io->out, io->scores,
                                            ctx->max_kv, ctx->profiling ? ctx->ev0 : nullptr,
@@ -1000,6 +1010,7 @@ void pa_destroy(pa_ctx* ctx) {
     ctx->items.release();
     for (auto& t : ctx->tables) t.release();
     ctx->table_pool.release();
+    ctx->alibi.release();
     ctx->step_staging.release();
     ctx->part_acc.release();
     ctx->part_ml.release();
@@ -1166,7 +1177,7 @@ void shape_tables(pa_ctx* ctx, bool shared) {
 size_t table_upload_bytes(pa_ctx* ctx, int32_t count, size_t* id_bytes, bool* with_descs) {
     *id_bytes = std::max<size_t>(((size_t)count * sizeof(int32_t) + 127) & ~(size_t)127, 128);
     size_t total = *id_bytes;
-    *with_descs = decode_u8_shape(ctx->cfg) && !ctx->h_dec.empty();
+    *with_descs = decode_u8_shape(ctx) && !ctx->h_dec.empty();
     if (*with_descs)
         for (int w = 0; w < 2; ++w) {
             ctx->desc_off[w] = total;
@@ -1290,6 +1301,7 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
             if (had) plan_items(ctx);
             return;
         }
+        PA_REQUIRE(!ctx->has_alibi, PA_NOT_IMPLEMENTED, "block-sparse prefill is not available with ALiBi slopes");
         PA_REQUIRE(mfma_shape(c) && c.block_size >= 32, PA_NOT_IMPLEMENTED,
                    "block-sparse prefill needs a block_size of 32 to 256 (a power of two), head_size 64 or 128 and a u8 cache "
                    "or one of the query's type");
@@ -1439,8 +1451,8 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         // a step of single-token sequences that all go to one of the decode kernels: it appends the new rows itself
         const bool fuse = ctx->step_ready &&
-                          ((decode_u8_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B) ||
-                           (mfma_shape(ctx->cfg) && decode16_shape(ctx->cfg) && (int32_t)ctx->h_dec16.size() == ctx->B &&
+                          ((decode_u8_shape(ctx) && (int32_t)ctx->h_dec.size() == ctx->B) ||
+                           (mfma_shape(ctx) && decode16_shape(ctx) && (int32_t)ctx->h_dec16.size() == ctx->B &&
                             ctx->n_sparse == 0 && ctx->n_single == ctx->n_items));
         if (fuse) check_io(ctx, layer, io, true, false);
         else do_kv_append(ctx, layer, io);
@@ -1550,6 +1562,30 @@ int32_t pa_rotation_data(const int64_t* evicted, int32_t num_evicted, int64_t nu
             }
         }
         *count = n;
+    });
+}
+
+int32_t pa_set_alibi_slopes(pa_ctx* ctx, const float* slopes, int32_t count) {
+    if (!ctx) return PA_INVALID_C_PARAM;
+    return guarded(ctx, [&] {
+        PA_REQUIRE(count == 0 || (slopes && count == ctx->cfg.num_heads), PA_PARAMETER_MISMATCH,
+                   "alibi_slopes must be empty or hold one slope per query head");
+        bool any = false;
+        for (int32_t h = 0; h < count; ++h) {
+            PA_REQUIRE(std::isfinite(slopes[h]), PA_PARAMETER_MISMATCH, "alibi_slopes must be finite");
+            any = any || slopes[h] != 0.0f;
+        }
+        HIP_CHECK(hipSetDevice(ctx->cfg.device));
+        HIP_CHECK(hipStreamSynchronize(ctx->stream));  // earlier launches may still read the old slopes
+        if (any) {
+            const size_t bytes = (size_t)count * sizeof(float);
+            ctx->alibi.reserve(bytes);
+            HIP_CHECK(hipMemcpyAsync(ctx->alibi.p, slopes, bytes, hipMemcpyHostToDevice, ctx->stream));
+            HIP_CHECK(hipStreamSynchronize(ctx->stream));  // `slopes` is the caller's, pageable
+        }
+        // the step's plan depends on which kernels serve it: a step that has begun has to begin again
+        if (any != ctx->has_alibi) ctx->step_ready = false;
+        ctx->has_alibi = any;
     });
 }
 

@@ -75,6 +75,12 @@ class PagedAttention:
         ids = _i32(block_indices)
         self._ck(L.lib().pa_set_block_indices(self._h, layer, _p32(ids), len(ids), int(num_blocks)))
 
+    def set_alibi_slopes(self, slopes):
+        """The op's `alibi_slopes` input: one f32 slope per query head (None or empty: no ALiBi term).  Call before
+        ``step_begin``; a context with slopes runs on the shape-generic kernels."""
+        a = np.ascontiguousarray(slopes if slopes is not None else [], dtype=np.float32)
+        self._ck(L.lib().pa_set_alibi_slopes(self._h, a.ctypes.data_as(C.POINTER(C.c_float)), len(a)))
+
     def set_block_indices_per_layer(self, tables, num_blocks, first_layer=0):
         """`block_indices.<L>` of layers first_layer .. first_layer + len(tables) - 1 in one call."""
         arrs = [_i32(t) for t in tables]

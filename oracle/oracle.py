@@ -188,6 +188,31 @@ def paged_attention_kv(query, q_dtype, key_cache, value_cache, k_dtype, v_dtype,
     return out, out16, scores
 
 
+def paged_attention_alibi(query, q_dtype, key_cache, value_cache, k_dtype, v_dtype, past_lens, subsequence_begins,
+                          block_indices, block_indices_begins, Hq, Hkv, Dk, Dv, bs, scale, alibi_slopes, sliding_window=0,
+                          score_aggregation_window=None, want_scores=True, num_threads=1):
+    """paged_attention_kv with the op's alibi_slopes input (f32 [Hq])."""
+    B = len(past_lens)
+    T = int(subsequence_begins[-1])
+    out = np.zeros((T, Hq * Dv), dtype=np.float32)
+    out16 = np.zeros((T, Hq * Dv), dtype=np.uint16)
+    total = int(np.sum(past_lens.astype(np.int64)) + T)
+    scores = np.zeros(total, dtype=np.float32) if want_scores else None
+    saw = None if score_aggregation_window is None else np.ascontiguousarray(score_aggregation_window, dtype=np.int32)
+    slopes = np.ascontiguousarray(alibi_slopes, dtype=np.float32)
+    assert slopes.shape == (Hq,)
+    rc = lib().orc_paged_attention_alibi(
+        _ptr(query, C.c_uint16), C.c_int32(q_dtype), _ptr(key_cache, C.c_uint8), _ptr(value_cache, C.c_uint8),
+        C.c_int32(k_dtype), C.c_int32(v_dtype), C.c_int64(key_cache.shape[0]), _ptr(past_lens, C.c_int32),
+        _ptr(subsequence_begins, C.c_int32), _ptr(block_indices, C.c_int32), _ptr(block_indices_begins, C.c_int32),
+        _ptr(saw, C.c_int32), C.c_int32(B), C.c_int32(Hq), C.c_int32(Hkv), C.c_int32(Dk), C.c_int32(Dv), C.c_int32(bs),
+        C.c_float(scale), C.c_int32(sliding_window), _ptr(slopes, C.c_float), _ptr(out, C.c_float), _ptr(out16, C.c_uint16),
+        _ptr(scores, C.c_float), C.c_int32(num_threads))
+    if rc != 0:
+        raise RuntimeError(_err())
+    return out, out16, scores
+
+
 def paged_attention(query, q_dtype, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,
                     block_indices, block_indices_begins, Hq, Hkv, D, bs, scale, sliding_window=0,
                     score_aggregation_window=None, want_scores=True, num_threads=1):

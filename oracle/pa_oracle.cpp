@@ -38,6 +38,8 @@
 //                            nibble first; pinned by the same closed-form invariants)
 //   orc_kv_append            PARITY UNPINNED vs the plugin (pinned by brute-force gather/scatter)
 //   orc_paged_attention      PARITY UNPINNED vs the plugin (pinned against textbook SDPA in float64)
+//   orc_paged_attention_alibi  PARITY UNPINNED vs the plugin (the op's alibi_slopes term: the paper's formula, bias
+//                            after the scaling; pinned against a float64 evaluation of it)
 //   orc_rotate_cache         PARITY UNPINNED vs the plugin (the re-rotation of cached K rows happens inside the op;
 //                            pinned by the closed form: RoPE at position p followed by the rotation for delta equals
 //                            RoPE at p - delta, and for u8 rows by the quantisation recipe above)
@@ -778,7 +780,8 @@ static int32_t paged_attention_impl(const uint16_t* query, int32_t q_dtype, cons
                             const int32_t* block_indices_begins, const int32_t* score_aggregation_window, int32_t B,
                             int32_t Hq, int32_t Hkv, int32_t D, int32_t bs, float scale, int32_t sliding_window,
                             float* out_f32, uint16_t* out16, float* scores, int32_t num_threads,
-                            const uint8_t* const* retained, int32_t xb, int32_t Dv = -1, int32_t v_dtype = -1) {
+                            const uint8_t* const* retained, int32_t xb, int32_t Dv = -1, int32_t v_dtype = -1,
+                            const float* alibi_slopes = nullptr) {
     if (Dv < 0) Dv = D;
     if (v_dtype < 0) v_dtype = cache_dtype;
     if (Hq % Hkv) { g_error = "Hq must be a multiple of Hkv"; return -14; }
@@ -842,6 +845,8 @@ static int32_t paged_attention_impl(const uint16_t* query, int32_t q_dtype, cons
 #pragma omp simd reduction(+ : s)
                         for (int d = 0; d < D; ++d) s += q[d] * kr[d];
                         s *= scale;
+                        // ALiBi: a bias linear in the distance to the query position, a slope per query head
+                        if (alibi_slopes) s += alibi_slopes[hq] * (float)(j - last);
                         p[j] = s;
                         m = std::fmax(m, s);
                     }
@@ -903,6 +908,24 @@ int32_t orc_paged_attention_kv(const uint16_t* query, int32_t q_dtype, const uin
                                 subsequence_begins, block_indices, block_indices_begins, score_aggregation_window, B, Hq,
                                 Hkv, Dk, bs, scale, sliding_window, out_f32, out16, scores, num_threads, nullptr, 0, Dv,
                                 v_dtype);
+}
+
+// ... and with the op's `alibi_slopes` input (input 11; f32 [Hq], empty for models without ALiBi): logit =
+// scale * q . k + slope[head] * (key position - query position).  PARITY UNPINNED vs OpenVINO: the term is applied
+// inside the op and the reference tree neither sets the input (a graph constant made by the SDPAToPagedAttention pass)
+// nor holds a vector for it; this is the ALiBi of the paper (arXiv 2108.12409), bias added after the scaling, pinned by
+// a float64 evaluation of that formula.
+int32_t orc_paged_attention_alibi(const uint16_t* query, int32_t q_dtype, const uint8_t* key_cache,
+                                  const uint8_t* value_cache, int32_t k_dtype, int32_t v_dtype, int64_t num_blocks,
+                                  const int32_t* past_lens, const int32_t* subsequence_begins,
+                                  const int32_t* block_indices, const int32_t* block_indices_begins,
+                                  const int32_t* score_aggregation_window, int32_t B, int32_t Hq, int32_t Hkv, int32_t Dk,
+                                  int32_t Dv, int32_t bs, float scale, int32_t sliding_window, const float* alibi_slopes,
+                                  float* out_f32, uint16_t* out16, float* scores, int32_t num_threads) {
+    return paged_attention_impl(query, q_dtype, key_cache, value_cache, k_dtype, num_blocks, past_lens,
+                                subsequence_begins, block_indices, block_indices_begins, score_aggregation_window, B, Hq,
+                                Hkv, Dk, bs, scale, sliding_window, out_f32, out16, scores, num_threads, nullptr, 0, Dv,
+                                v_dtype, alibi_slopes);
 }
 
 // ------------------------------------------------------------------ XAttention (sparse prefill, importance estimate)

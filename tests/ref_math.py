@@ -70,11 +70,11 @@ def dequant_rows_u4(rows):
     return (codes.astype(np.float32) - zp) * scale
 
 
-def attention_f64(q, K, V, past, scale, sliding_window, W):
+def attention_f64(q, K, V, past, scale, sliding_window, W, slopes=None):
     """Textbook attention in float64 for one sequence and one kv head.
 
     q [q_len, G, D], K [kv_len, D], V [kv_len, Dv] -> out [q_len, G, Dv], scores [kv_len] (sum over G heads and
-    last W rows).
+    last W rows).  slopes [G]: ALiBi, logit += slope * (key position - query position).
     """
     q = q.astype(np.float64)
     K = K.astype(np.float64)
@@ -87,6 +87,8 @@ def attention_f64(q, K, V, past, scale, sliding_window, W):
         last = past + i
         first = max(0, last + 1 - sliding_window) if sliding_window > 0 else 0
         s = (q[i] @ K[first:last + 1].T) * scale  # [G, n]
+        if slopes is not None:
+            s = s + np.asarray(slopes, np.float64)[:, None] * (np.arange(first, last + 1) - last)[None, :]
         s -= s.max(axis=1, keepdims=True)
         p = np.exp(s)
         p /= p.sum(axis=1, keepdims=True)

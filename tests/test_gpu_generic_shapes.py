@@ -85,3 +85,71 @@ def test_refused_configurations(pkg):
         hs = kw.pop("head_size")
         with pytest.raises(pkg.PaError):
             pkg.PagedAttention(8, 2, hs, 32, "f16", "u8", **kw)
+
+
+ALIBI = [
+    # (query type, Dk, Dv, key cache type, value cache type, block size, Hq, Hkv): tuned shapes (which a context with
+    # slopes leaves for the shape-generic kernels) and others
+    ("f16", 128, 128, "u8", "u8", 32, 8, 2), ("bf16", 128, 128, "bf16", "bf16", 32, 28, 4), ("f16", 64, 64, "f16", "f16", 16, 4, 4),
+    ("bf16", 96, 96, "u8", "u8", 32, 6, 2), ("f16", 128, 64, "u4", "f16", 32, 8, 1),
+]
+
+
+@pytest.mark.parametrize("qd,Dk,Dv,kd,vd,bs,Hq,Hkv", ALIBI)
+@pytest.mark.parametrize("kind", ["mixed", "decode"])
+def test_alibi_slopes(pkg, qd, Dk, Dv, kd, vd, bs, Hq, Hkv, kind):
+    """The op's alibi_slopes input: outputs and scores against the checker's form with slopes; with all-zero slopes
+    and after taking the slopes away again the context is back on its own kernels with their results."""
+    import torch
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(Dk * 17 + Hq)
+    past, new = ([0, 45, 700, 9], [37, 1, 1, 70]) if kind == "mixed" else ([300, 5, 1500], [1, 1, 1])
+    print(f"case alibi {qd} Dk{Dk} Dv{Dv} {kd}/{vd} bs{bs} {kind}", flush=True)
+    c = _case(rng, qd, Dk, Dv, kd, vd, bs, Hq, Hkv, past, new)
+    W = np.minimum(c["new"], 2).astype(np.int32)
+    sw = 0 if kind == "mixed" else 600
+    scale = float(1.0 / np.sqrt(Dk))
+    # slopes of the paper's geometric kind, one head without a slope
+    slopes = (2.0 ** -(8.0 * (np.arange(Hq) + 1) / Hq)).astype(np.float32)
+    slopes[Hq // 2] = 0.0
+    kc_ref, vc_ref = c["kc"].copy(), c["vc"].copy()
+    O.kv_append_kv(c["k"], c["v"], c["qdt"], kc_ref, vc_ref, c["kdt"], c["vdt"], c["past"], c["sb"], c["table"], c["bib"],
+                   Hkv, Dk, Dv, bs)
+    ref_out, _, ref_sc = O.paged_attention_alibi(c["q"], c["qdt"], kc_ref, vc_ref, c["kdt"], c["vdt"], c["past"], c["sb"],
+                                                 c["table"], c["bib"], Hq, Hkv, Dk, Dv, bs, scale, slopes, sw, W, True, 8)
+    plain_out, _, plain_sc = O.paged_attention_kv(c["q"], c["qdt"], kc_ref, vc_ref, c["kdt"], c["vdt"], c["past"], c["sb"],
+                                                  c["table"], c["bib"], Hq, Hkv, Dk, Dv, bs, scale, sw, W, True, 8)
+    assert np.abs(ref_out - plain_out).max() > 1e-2   # (the slopes matter on this data)
+    op = pkg.PagedAttention(Hq, Hkv, Dk, bs, qd, kd, 1, 0, torch.cuda.current_stream(dev), v_head_size=Dv,
+                            value_cache_dtype=vd)
+    q, k, v = (H.to_device_16(torch, c[n], qd, dev) for n in ("q", "k", "v"))
+
+    def run(want):
+        kc, vc = torch.from_numpy(c["kc"]).to(dev), torch.from_numpy(c["vc"]).to(dev)
+        out = torch.zeros(q.shape[0], Hq * Dv, dtype=q.dtype, device=dev)
+        op.step_begin(c["past"], c["sb"], c["bib"], int((c["past"] + c["new"]).max()), W, sw, scale)
+        op.set_block_indices(c["table"], c["pool"])
+        scores = torch.full((op.total_scores,), float("nan"), dtype=torch.float32, device=dev)
+        op.forward(q, k, v, kc, vc, out, scores)
+        op.synchronize()
+        assert np.array_equal(kc.cpu().numpy(), kc_ref) and np.array_equal(vc.cpu().numpy(), vc_ref), "cache bytes differ"
+        H.assert_close(out.float().cpu().numpy(), want[0], qd)
+        H.assert_close(scores.cpu().numpy(), want[1], "f16", "scores")
+        return out.view(torch.int16).cpu().numpy(), scores.cpu().numpy()
+
+    before = run((plain_out, plain_sc))
+    op.set_alibi_slopes(slopes)
+    with pytest.raises(pkg.PaError):   # the step's plan is void after the change: it has to begin again
+        op.attention(q, torch.from_numpy(c["kc"]).to(dev), torch.from_numpy(c["vc"]).to(dev),
+                     torch.zeros(q.shape[0], Hq * Dv, dtype=q.dtype, device=dev))
+    run((ref_out, ref_sc))
+    op.set_alibi_slopes(np.zeros(Hq, np.float32))
+    after = run((plain_out, plain_sc))
+    assert np.array_equal(before[0], after[0]) and np.array_equal(before[1], after[1])
+    op.set_alibi_slopes(slopes)
+    run((ref_out, ref_sc))
+    op.set_alibi_slopes(None)
+    after = run((plain_out, plain_sc))
+    assert np.array_equal(before[0], after[0])
+    with pytest.raises(pkg.PaError):   # one slope per query head
+        op.set_alibi_slopes(slopes[:-1])

@@ -214,6 +214,25 @@ def test_attention_with_a_head_size_and_type_per_tensor_matches_float64(Dk, Dv, 
             np.testing.assert_allclose(got, o, rtol=2e-5, atol=2e-5)
             sc_ref += s
         np.testing.assert_allclose(scores[so[b]:so[b + 1]], sc_ref, rtol=2e-5, atol=2e-5)
+    # ... with the op's alibi_slopes input: logit += slope[head] * (key position - query position), against the
+    # float64 form; with a sliding window on top; zero slopes give the bits of the form without slopes
+    slopes = (2.0 ** -(np.arange(Hq) * 8.0 / Hq + 1)).astype(np.float32) * np.where(np.arange(Hq) % 3 == 2, 0.0, 1.0).astype(np.float32)
+    for sw in (0, 13):
+        out_a, _, scores_a = O.paged_attention_alibi(q, qdt, kc, vc, kdt, vdt, past, sb, table, bib, Hq, Hkv, Dk, Dv, bs,
+                                                     scale, slopes, sw, W, True, 4)
+        assert np.abs(out_a - out).max() > 1e-3   # (the slopes matter on this data)
+        for b in range(B):
+            sc_ref = np.zeros(int(tot[b]))
+            for h in range(Hkv):
+                o, s = R.attention_f64(qf[sb[b]:sb[b + 1], h * G:(h + 1) * G], rows(kc, Dk, kdt, b, h),
+                                       rows(vc, Dv, vdt, b, h), int(past[b]), scale, sw, int(W[b]), slopes[h * G:(h + 1) * G])
+                got = out_a[sb[b]:sb[b + 1]].reshape(-1, Hq, Dv)[:, h * G:(h + 1) * G]
+                np.testing.assert_allclose(got, o, rtol=2e-5, atol=2e-5)
+                sc_ref += s
+            np.testing.assert_allclose(scores_a[so[b]:so[b + 1]], sc_ref, rtol=2e-5, atol=2e-5)
+    out_z, out16_z, scores_z = O.paged_attention_alibi(q, qdt, kc, vc, kdt, vdt, past, sb, table, bib, Hq, Hkv, Dk, Dv, bs,
+                                                       scale, np.zeros(Hq, np.float32), 0, W, True, 4)
+    assert np.array_equal(out16_z, out16) and np.array_equal(scores_z, scores)
     # ... and equal head sizes and types give the bits of the plain form
     if Dk == Dv and kdt == vdt and kdt != O.DT_U4:
         out2, out16_2, scores2 = O.paged_attention(q, qdt, kc, vc, kdt, past, sb, table, bib, Hq, Hkv, Dk, bs, scale, 0, W,

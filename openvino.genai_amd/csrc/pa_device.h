@@ -185,6 +185,14 @@ constexpr int GENERIC_MAX_HEAD_SIZE = 512;
 struct GenericShape {
     int32_t Hq, Hkv, Dk, Dv, bs, kdt, vdt;
 };
+// Query heads one wave of the shape-generic attention kernel serves (1, 2, 4 or 8): heads of one kv head's group, as
+// many as keep the wave's query rows within 8 KB of LDS.
+inline int generic_heads_per_wave(const GenericShape& sh) {
+    const int G = sh.Hq / sh.Hkv;
+    int gc = 1;
+    while (gc < 8 && gc < G && 2 * gc * sh.Dk <= 2048) gc *= 2;
+    return gc;
+}
 hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype,
                                     const void* query, const void* key_cache, const void* value_cache,
                                     const int32_t* block_indices, const AttnWorkspace& ws, void* out, float* scores,

@@ -3,9 +3,9 @@
 // (`f32 scale | f32 zero-point | D codes`) or u4 rows (`f32 scale | f32 zero-point | D / 2 bytes`, element 2 i in the
 // high nibble of byte i).  Everything the tuned kernels do not take runs here.
 //
-// pa_generic_kernel     : one wave per (token, query head, split).  Lanes take consecutive KV positions for QK (each
-//                         lane owns one cache row), then the wave walks the 64 positions with lanes across the value
-//                         head for PV.  Online softmax per wave.
+// pa_generic_kernel     : one wave per (token, kv head, up to eight query heads of its group, split).  Lanes take
+//                         consecutive KV positions for QK (each lane owns one cache row, read once for all the heads),
+//                         then regroup across the value head for PV.  Online softmax per head and wave.
 // pa_merge_kernel       : folds the split partials (m, l, acc) into the output row and keeps the final
 //                         (max, denominator) of every (token, head) for the score kernels.
 // pa_scores_single      : scores of single-token (decode) sequences from the stored logits.
@@ -63,6 +63,28 @@ struct RowReader {
             }
         }
     }
+    // eight consecutive elements as stored: the codes of u8 / u4 rows (the element is (code - zp) * scale), the values
+    // of 16-bit rows (scale 1, zero-point 0)
+    __device__ void load8_codes(int d, float* out) const {
+        if (dt == DT_U8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(row + d);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                out[e] = (float)((v.x >> (8 * e)) & 0xff);
+                out[4 + e] = (float)((v.y >> (8 * e)) & 0xff);
+            }
+        } else if (dt == DT_U4) {
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(row + d / 2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t byte = (v >> (8 * e)) & 0xff;
+                out[2 * e] = (float)(byte >> 4);
+                out[2 * e + 1] = (float)(byte & 15);
+            }
+        } else {
+            load8(d, out);
+        }
+    }
     __device__ float load1(int d) const {
         if (dt == DT_U8) return ((float)row[d] - zp) * scale;
         if (dt == DT_U4) {
@@ -74,29 +96,51 @@ struct RowReader {
     }
 };
 
-template <int QDT>
-__global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, GenericShape sh, const uint16_t* __restrict__ query,
+// One wave per (token, kv head, set of GC query heads of its group, split): every cache row it touches serves all GC
+// heads.  QK: a lane owns a position, walks its key row eight elements at a time against the heads' query rows (scaled,
+// f32, in LDS: all lanes read the same words).  PV: the lanes regroup -- LPR lanes to a value row, eight channels each,
+// 64 / LPR rows per step -- and fetch the rows' probabilities from the lanes that own them; the row groups' partial
+// sums are added once at the end.  Online softmax per head and wave.
+template <int QDT, int GC>
+__global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDev st, GenericShape sh, const uint16_t* __restrict__ query,
                                                          const uint8_t* __restrict__ key_cache,
                                                          const uint8_t* __restrict__ value_cache,
                                                          const int32_t* __restrict__ block_indices, AttnWorkspace ws,
                                                          int store_logits) {
-    constexpr int EPL = MAX_D / 64;  // value channels per lane at most
-    __shared__ float qs[4][MAX_D];
+    extern __shared__ float qs_all[];  // [4 waves][GC][Dk]
     const int lane = threadIdx.x & 63;
     const int wv = threadIdx.x >> 6;
     const int Dk = sh.Dk, Dv = sh.Dv;
+    const int G = sh.Hq / sh.Hkv;
+    const int sets = ceil_div(G, GC);
     const long wave = (long)blockIdx.x * 4 + wv;
-    const long total = (long)st.T * sh.Hq * ws.nsplit;
+    const long total = (long)st.T * sh.Hkv * sets * ws.nsplit;
     const bool valid = wave < total;
-    int split = 0, hq = 0, t = 0;
+    float* qs = qs_all + (long)wv * GC * Dk;
+    int split = 0, hkv = 0, t = 0, g0 = 0, ng = 0;
     if (valid) {
         split = (int)(wave % ws.nsplit);
-        hq = (int)((wave / ws.nsplit) % sh.Hq);
-        t = (int)(wave / ((long)ws.nsplit * sh.Hq));
-        for (int d = lane; d < Dk; d += 64) qs[wv][d] = load16<QDT>(query[((long)t * sh.Hq + hq) * Dk + d]) * st.scale;
+        const int set = (int)((wave / ws.nsplit) % sets);
+        hkv = (int)((wave / ((long)ws.nsplit * sets)) % sh.Hkv);
+        t = (int)(wave / ((long)ws.nsplit * sets * sh.Hkv));
+        g0 = set * GC;
+        ng = min(GC, G - g0);
+        for (int idx = lane; idx < GC * Dk; idx += 64) {
+            const int g = idx / Dk, d = idx - g * Dk;
+            qs[idx] = g < ng ? load16<QDT>(query[((long)t * sh.Hq + hkv * G + g0 + g) * Dk + d]) * st.scale : 0.0f;
+        }
     }
     __syncthreads();
     if (!valid) return;
+    // Quantised rows are multiplied as codes; scale and zero-point come in once per row:
+    //   q . k = scale_k (q . codes - zp_k sum(q)),   sum_j p_j v_j = sum_j (p_j scale_v) codes_j - sum_j p_j scale_v zp_v
+    float qsum[GC];
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        float part = 0.0f;
+        for (int d = lane; d < Dk; d += 64) part += qs[g * Dk + d];
+        qsum[g] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wave_sum(part))));  // (the same in every lane)
+    }
 
     const int b = st.token_seq[t];
     const int i = t - st.subsequence_begins[b];
@@ -108,60 +152,114 @@ __global__ __launch_bounds__(256) void pa_generic_kernel(StepDev st, GenericShap
     const int chunk = ceil_div(ceil_div(n, ws.nsplit), 64) * 64;
     const int j_begin = first + split * chunk;
     const int j_end = min(last + 1, j_begin + chunk);
-    const int hkv = hq / (sh.Hq / sh.Hkv);
     const int32_t* table = block_indices + st.block_indices_begins[b];
     const bool keep_logits = store_logits && q_len == 1 && st.score_window[b] > 0;
-    float* logit_row = ws.logits + (long)hq * ws.total_scores + st.score_offsets[b];
-    const float slope = ws.alibi ? ws.alibi[hq] : 0.0f;
-
-    float m = -INFINITY, l = 0.0f;
-    float acc[EPL];
+    const int hq0 = hkv * G + g0;
+    float slope[GC];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
+    for (int g = 0; g < GC; ++g) slope[g] = ws.alibi && g < ng ? ws.alibi[hq0 + g] : 0.0f;
+
+    // value rows: LPR lanes to a row (a power of two, at least Dv / 8), RPS rows per step
+    int lpr = 1;
+    while (lpr * 8 < Dv) lpr <<= 1;
+    const int rps = 64 / lpr;
+    const int vlane = lane & (lpr - 1), vrow = lane / lpr;
+    const bool v_active = 8 * vlane < Dv;
+
+    float m[GC], l[GC], acc[GC][8], zacc[GC];
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+        zacc[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
+    }
 
     for (int j0 = j_begin; j0 < j_end; j0 += 64) {
         const int j = j0 + lane;
         const bool live = j < j_end;
         long phys = 0;
-        float s = -INFINITY;
+        float sc[GC];
+#pragma unroll
+        for (int g = 0; g < GC; ++g) sc[g] = 0.0f;
         if (live) {
             phys = table[j / sh.bs];
             RowReader kr(key_cache, phys, hkv, j % sh.bs, sh.Hkv, sh.bs, Dk, sh.kdt);
-            float dot = 0.0f;
             for (int d = 0; d < Dk; d += 8) {
                 float k8[8];
-                kr.load8(d, k8);
+                kr.load8_codes(d, k8);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) dot += qs[wv][d + e] * k8[e];
+                for (int g = 0; g < GC; ++g) {
+                    const float* qg = qs + g * Dk + d;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sc[g] += qg[e] * k8[e];
+                }
             }
-            s = ws.alibi ? dot + slope * (float)(j - last) : dot;
-            if (keep_logits) logit_row[j] = s;
-        }
-        const float m_new = fmaxf(m, wave_max(s));
-        const float corr = (m == -INFINITY) ? 0.0f : __expf(m - m_new);
-        const float p = live ? __expf(s - m_new) : 0.0f;
-        l = l * corr + wave_sum(p);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] *= corr;
-        m = m_new;
+            for (int g = 0; g < GC; ++g) sc[g] = kr.scale * (sc[g] - kr.zp * qsum[g]);
+        }
+        float p[GC];
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            float x = -INFINITY;
+            if (live) {
+                x = ws.alibi ? sc[g] + slope[g] * (float)(j - last) : sc[g];
+                if (keep_logits && g < ng) ws.logits[(long)(hq0 + g) * ws.total_scores + st.score_offsets[b] + j] = x;
+            }
+            const float m_new = fmaxf(m[g], wave_max(x));
+            const float corr = (m[g] == -INFINITY) ? 0.0f : __expf(m[g] - m_new);
+            p[g] = live ? __expf(x - m_new) : 0.0f;
+            l[g] = l[g] * corr + wave_sum(p[g]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] *= corr;
+            zacc[g] *= corr;
+            m[g] = m_new;
+        }
         const int cnt = min(64, j_end - j0);
-        for (int jj = 0; jj < cnt; ++jj) {
-            const float pj = __shfl(p, jj, WAVE);
-            const long pb = __shfl(phys, jj, WAVE);
-            RowReader vr(value_cache, pb, hkv, (j0 + jj) % sh.bs, sh.Hkv, sh.bs, Dv, sh.vdt);
+        for (int r = 0; r * rps < cnt; ++r) {
+            const int jj = r * rps + vrow;            // the row of this lane's group in this step
+            const int src = min(jj, 63);
+            const long pb = __shfl(phys, src, WAVE);
+            float pj[GC];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e)
-                if (lane + 64 * e < Dv) acc[e] += pj * vr.load1(lane + 64 * e);
+            for (int g = 0; g < GC; ++g) pj[g] = __shfl(p[g], src, WAVE);
+            if (v_active && jj < cnt) {
+                RowReader vr(value_cache, pb, hkv, (j0 + jj) % sh.bs, sh.Hkv, sh.bs, Dv, sh.vdt);
+                float v8[8];
+                vr.load8_codes(8 * vlane, v8);
+#pragma unroll
+                for (int g = 0; g < GC; ++g) {
+                    const float w = pj[g] * vr.scale;
+                    zacc[g] += w * vr.zp;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[g][e] += w * v8[e];
+                }
+            }
         }
     }
-    const long slot = ((long)t * sh.Hq + hq) * ws.nsplit + split;
-    if (lane == 0) {
-        ws.part_ml[2 * slot] = m;
-        ws.part_ml[2 * slot + 1] = l;
-    }
+    // the zero-point terms of the lane's rows, then the row groups' partial sums: lanes with the same channels add up
 #pragma unroll
-    for (int e = 0; e < EPL; ++e)
-        if (lane + 64 * e < Dv) ws.part_acc[slot * Dv + lane + 64 * e] = acc[e];
+    for (int g = 0; g < GC; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[g][e] -= zacc[g];
+            for (int o = lpr; o < 64; o <<= 1) acc[g][e] += __shfl_xor(acc[g][e], o, WAVE);
+        }
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        if (g >= ng) break;
+        const long slot = ((long)t * sh.Hq + hq0 + g) * ws.nsplit + split;
+        if (lane == 0) {
+            ws.part_ml[2 * slot] = m[g];
+            ws.part_ml[2 * slot + 1] = l[g];
+        }
+        if (vrow == 0 && v_active) {
+            float* dst = ws.part_acc + slot * Dv + 8 * vlane;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dst[e] = acc[g][e];
+        }
+    }
 }
 
 template <int QDT>
@@ -342,14 +440,21 @@ template <int QDT>
 hipError_t launch_typed(hipStream_t s, const StepDev& st, const GenericShape& sh, const void* query, const void* kc,
                         const void* vc, const int32_t* bi, const AttnWorkspace& ws, void* out, float* scores,
                         int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1) {
-    const long waves = (long)st.T * sh.Hq * ws.nsplit;
+    const int gc = generic_heads_per_wave(sh);
+    const long waves = (long)st.T * sh.Hkv * ceil_div(sh.Hq / sh.Hkv, gc) * ws.nsplit;
     if (waves == 0) return hipSuccess;
     auto q = reinterpret_cast<const uint16_t*>(query);
     auto k = reinterpret_cast<const uint8_t*>(kc);
     auto v = reinterpret_cast<const uint8_t*>(vc);
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    const size_t lds = (size_t)4 * gc * sh.Dk * sizeof(float);
     if (ev0) (void)hipEventRecord(ev0, s);
-    hipLaunchKernelGGL((pa_generic_kernel<QDT>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, st, sh, q, k, v, bi, ws,
-                       scores ? 1 : 0);
+    switch (gc) {
+        case 1: hipLaunchKernelGGL((pa_generic_kernel<QDT, 1>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
+        case 2: hipLaunchKernelGGL((pa_generic_kernel<QDT, 2>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
+        case 4: hipLaunchKernelGGL((pa_generic_kernel<QDT, 4>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
+        default: hipLaunchKernelGGL((pa_generic_kernel<QDT, 8>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
+    }
     if (ev1) (void)hipEventRecord(ev1, s);
     const long rows = (long)st.T * sh.Hq;
     hipLaunchKernelGGL((pa_merge_kernel<QDT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, st, sh, ws,

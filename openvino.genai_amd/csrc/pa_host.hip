@@ -1127,7 +1127,10 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         ctx->h_sb.assign(sb, sb + B + 1);
         ctx->h_bib.assign(bib, bib + B + 1);
         // split-K plan: enough waves to fill 256 CUs several times over, at least 256 positions per split
-        const int64_t rows = (int64_t)T * ctx->cfg.num_heads;
+        // (a wave of the shape-generic kernel serves up to eight heads of a kv head's group)
+        const pa::GenericShape gsh = generic_shape_of(ctx->cfg);
+        const int gc = pa::generic_heads_per_wave(gsh);
+        const int64_t rows = (int64_t)T * gsh.Hkv * pa::ceil_div(gsh.Hq / gsh.Hkv, gc);
         const int32_t eff_kv = m->sliding_window > 0 ? std::min(max_kv, m->sliding_window) : max_kv;
         int64_t want = (4096 + rows - 1) / rows;
         int64_t cap = std::max<int64_t>(1, eff_kv / 256);

@@ -149,6 +149,9 @@ struct StepDev {
     const int32_t* score_window;          // [B], already clamped to [0, q_len]
     const int32_t* score_offsets;         // [B+1] prefix sum of past+new
     const int32_t* token_seq;             // [T] sequence of each token
+    const int32_t* gtiles;                // [n_gtiles] token tiles of the shape-generic attention kernel: up to eight
+                                          // consecutive tokens of one sequence, first token * 8 + (count - 1)
+    int32_t n_gtiles;
     int32_t B, T;
     int32_t sliding_window;
     float scale;
@@ -185,13 +188,23 @@ constexpr int GENERIC_MAX_HEAD_SIZE = 512;
 struct GenericShape {
     int32_t Hq, Hkv, Dk, Dv, bs, kdt, vdt;
 };
-// Query heads one wave of the shape-generic attention kernel serves (1, 2, 4 or 8): heads of one kv head's group, as
-// many as keep the wave's query rows within 8 KB of LDS.
-inline int generic_heads_per_wave(const GenericShape& sh) {
+// What one wave of the shape-generic attention kernel serves: `rows` (1, 2, 4 or 8) query rows that share every cache
+// row it reads -- `heads` heads of one kv head's group (a power of two) for each of `tokens` consecutive tokens of one
+// sequence -- as many as keep the wave's query rows within 8 KB of LDS.  Steps without multi-token sequences take one
+// token per wave.
+struct GenericPlan {
+    int rows, heads, tokens;
+};
+inline GenericPlan generic_plan(const GenericShape& sh, bool multi_token) {
     const int G = sh.Hq / sh.Hkv;
-    int gc = 1;
-    while (gc < 8 && gc < G && 2 * gc * sh.Dk <= 2048) gc *= 2;
-    return gc;
+    int most = 8;
+    while (most > 1 && most * sh.Dk > 1024) most >>= 1;
+    GenericPlan p;
+    p.heads = 1;
+    while (p.heads < most && p.heads < G) p.heads <<= 1;
+    p.tokens = multi_token ? most / p.heads : 1;
+    p.rows = p.heads * p.tokens;
+    return p;
 }
 hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype,
                                     const void* query, const void* key_cache, const void* value_cache,

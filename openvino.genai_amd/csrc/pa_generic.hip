@@ -3,9 +3,10 @@
 // (`f32 scale | f32 zero-point | D codes`) or u4 rows (`f32 scale | f32 zero-point | D / 2 bytes`, element 2 i in the
 // high nibble of byte i).  Everything the tuned kernels do not take runs here.
 //
-// pa_generic_kernel     : one wave per (token, kv head, up to eight query heads of its group, split).  Lanes take
-//                         consecutive KV positions for QK (each lane owns one cache row, read once for all the heads),
-//                         then regroup across the value head for PV.  Online softmax per head and wave.
+// pa_generic_kernel     : one wave per (tile of consecutive tokens of a sequence, kv head, heads of its group, split): up
+//                         to eight query rows.  Lanes take consecutive KV positions for QK (each lane owns one cache
+//                         row, read once for all the rows), then regroup across the value head for PV.  Online softmax
+//                         per query row and wave.
 // pa_merge_kernel       : folds the split partials (m, l, acc) into the output row and keeps the final
 //                         (max, denominator) of every (token, head) for the score kernels.
 // pa_scores_single      : scores of single-token (decode) sequences from the stored logits.
@@ -96,38 +97,43 @@ struct RowReader {
     }
 };
 
-// One wave per (token, kv head, set of GC query heads of its group, split): every cache row it touches serves all GC
-// heads.  QK: a lane owns a position, walks its key row eight elements at a time against the heads' query rows (scaled,
-// f32, in LDS: all lanes read the same words).  PV: the lanes regroup -- LPR lanes to a value row, eight channels each,
-// 64 / LPR rows per step -- and fetch the rows' probabilities from the lanes that own them; the row groups' partial
-// sums are added once at the end.  Online softmax per head and wave.
+// One wave per (token tile, kv head, set of heads of its group, split): GC query rows -- `hs` heads for each of the
+// tile's GC / hs consecutive tokens of one sequence -- share every cache row the wave touches.  QK: a lane owns a
+// position, walks its key row eight elements at a time against the query rows (scaled, f32, in LDS: all lanes read the
+// same words); each row masks what its token may not see.  PV: the lanes regroup -- LPR lanes to a value row, eight
+// channels each, 64 / LPR rows per step -- and fetch the rows' probabilities from the lanes that own them; the row
+// groups' partial sums are added once at the end.  Online softmax per query row and wave.
 template <int QDT, int GC>
 __global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDev st, GenericShape sh, const uint16_t* __restrict__ query,
                                                          const uint8_t* __restrict__ key_cache,
                                                          const uint8_t* __restrict__ value_cache,
                                                          const int32_t* __restrict__ block_indices, AttnWorkspace ws,
-                                                         int store_logits) {
+                                                         int store_logits, int hs) {
     extern __shared__ float qs_all[];  // [4 waves][GC][Dk]
     const int lane = threadIdx.x & 63;
     const int wv = threadIdx.x >> 6;
     const int Dk = sh.Dk, Dv = sh.Dv;
     const int G = sh.Hq / sh.Hkv;
-    const int sets = ceil_div(G, GC);
+    const int sets = ceil_div(G, hs);
     const long wave = (long)blockIdx.x * 4 + wv;
-    const long total = (long)st.T * sh.Hkv * sets * ws.nsplit;
+    const long total = (long)st.n_gtiles * sh.Hkv * sets * ws.nsplit;
     const bool valid = wave < total;
     float* qs = qs_all + (long)wv * GC * Dk;
-    int split = 0, hkv = 0, t = 0, g0 = 0, ng = 0;
+    int split = 0, hkv = 0, t0 = 0, nt = 0, g0 = 0, ng = 0;
     if (valid) {
         split = (int)(wave % ws.nsplit);
         const int set = (int)((wave / ws.nsplit) % sets);
         hkv = (int)((wave / ((long)ws.nsplit * sets)) % sh.Hkv);
-        t = (int)(wave / ((long)ws.nsplit * sets * sh.Hkv));
-        g0 = set * GC;
-        ng = min(GC, G - g0);
+        const int tile = st.gtiles[wave / ((long)ws.nsplit * sets * sh.Hkv)];
+        t0 = tile >> 3;          // the tile's first token
+        nt = (tile & 7) + 1;     // its tokens
+        g0 = set * hs;
+        ng = min(hs, G - g0);
+        // row r = (token t0 + r / hs, head g0 + r % hs); rows beyond the tile or the group are zero and write nothing
         for (int idx = lane; idx < GC * Dk; idx += 64) {
-            const int g = idx / Dk, d = idx - g * Dk;
-            qs[idx] = g < ng ? load16<QDT>(query[((long)t * sh.Hq + hkv * G + g0 + g) * Dk + d]) * st.scale : 0.0f;
+            const int r = idx / Dk, d = idx - r * Dk;
+            const int ti = r / hs, g = r - ti * hs;
+            qs[idx] = (ti < nt && g < ng) ? load16<QDT>(query[((long)(t0 + ti) * sh.Hq + hkv * G + g0 + g) * Dk + d]) * st.scale : 0.0f;
         }
     }
     __syncthreads();
@@ -136,28 +142,37 @@ __global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDe
     //   q . k = scale_k (q . codes - zp_k sum(q)),   sum_j p_j v_j = sum_j (p_j scale_v) codes_j - sum_j p_j scale_v zp_v
     float qsum[GC];
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
+    for (int r = 0; r < GC; ++r) {
         float part = 0.0f;
-        for (int d = lane; d < Dk; d += 64) part += qs[g * Dk + d];
-        qsum[g] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wave_sum(part))));  // (the same in every lane)
+        for (int d = lane; d < Dk; d += 64) part += qs[r * Dk + d];
+        qsum[r] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wave_sum(part))));  // (the same in every lane)
     }
 
-    const int b = st.token_seq[t];
-    const int i = t - st.subsequence_begins[b];
+    const int b = st.token_seq[t0];
+    const int i0 = t0 - st.subsequence_begins[b];
     const int q_len = st.subsequence_begins[b + 1] - st.subsequence_begins[b];
     const int past = st.past_lens[b];
-    const int last = past + i;
-    const int first = st.sliding_window > 0 ? max(0, last + 1 - st.sliding_window) : 0;
-    const int n = last + 1 - first;
+    const int sw = st.sliding_window;
+    // what the tile's tokens see together: from the first token's first position to the last token's own
+    const int last_w = past + i0 + nt - 1;
+    const int first_w = sw > 0 ? max(0, past + i0 + 1 - sw) : 0;
+    const int n = last_w + 1 - first_w;
     const int chunk = ceil_div(ceil_div(n, ws.nsplit), 64) * 64;
-    const int j_begin = first + split * chunk;
-    const int j_end = min(last + 1, j_begin + chunk);
+    const int j_begin = first_w + split * chunk;
+    const int j_end = min(last_w + 1, j_begin + chunk);
     const int32_t* table = block_indices + st.block_indices_begins[b];
     const bool keep_logits = store_logits && q_len == 1 && st.score_window[b] > 0;
     const int hq0 = hkv * G + g0;
     float slope[GC];
+    int row_last[GC], row_first[GC];  // the positions row r sees: [row_first, row_last]; none for rows that do not exist
 #pragma unroll
-    for (int g = 0; g < GC; ++g) slope[g] = ws.alibi && g < ng ? ws.alibi[hq0 + g] : 0.0f;
+    for (int r = 0; r < GC; ++r) {
+        const int ti = r / hs, g = r - ti * hs;
+        const bool exists = ti < nt && g < ng;
+        slope[r] = ws.alibi && exists ? ws.alibi[hq0 + g] : 0.0f;
+        row_last[r] = exists ? past + i0 + ti : -1;
+        row_first[r] = sw > 0 ? max(0, past + i0 + ti + 1 - sw) : 0;
+    }
 
     // value rows: LPR lanes to a row (a power of two, at least Dv / 8), RPS rows per step
     int lpr = 1;
@@ -168,12 +183,12 @@ __global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDe
 
     float m[GC], l[GC], acc[GC][8], zacc[GC];
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-        m[g] = -INFINITY;
-        l[g] = 0.0f;
-        zacc[g] = 0.0f;
+    for (int r = 0; r < GC; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.0f;
+        zacc[r] = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
+        for (int e = 0; e < 8; ++e) acc[r][e] = 0.0f;
     }
 
     for (int j0 = j_begin; j0 < j_end; j0 += 64) {
@@ -182,7 +197,7 @@ __global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDe
         long phys = 0;
         float sc[GC];
 #pragma unroll
-        for (int g = 0; g < GC; ++g) sc[g] = 0.0f;
+        for (int r = 0; r < GC; ++r) sc[r] = 0.0f;
         if (live) {
             phys = table[j / sh.bs];
             RowReader kr(key_cache, phys, hkv, j % sh.bs, sh.Hkv, sh.bs, Dk, sh.kdt);
@@ -190,74 +205,75 @@ __global__ __launch_bounds__(256, GC <= 4 ? 4 : 2) void pa_generic_kernel(StepDe
                 float k8[8];
                 kr.load8_codes(d, k8);
 #pragma unroll
-                for (int g = 0; g < GC; ++g) {
-                    const float* qg = qs + g * Dk + d;
+                for (int r = 0; r < GC; ++r) {
+                    const float* qr = qs + r * Dk + d;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) sc[g] += qg[e] * k8[e];
+                    for (int e = 0; e < 8; ++e) sc[r] += qr[e] * k8[e];
                 }
             }
 #pragma unroll
-            for (int g = 0; g < GC; ++g) sc[g] = kr.scale * (sc[g] - kr.zp * qsum[g]);
+            for (int r = 0; r < GC; ++r) sc[r] = kr.scale * (sc[r] - kr.zp * qsum[r]);
         }
         float p[GC];
 #pragma unroll
-        for (int g = 0; g < GC; ++g) {
+        for (int r = 0; r < GC; ++r) {
             float x = -INFINITY;
-            if (live) {
-                x = ws.alibi ? sc[g] + slope[g] * (float)(j - last) : sc[g];
-                if (keep_logits && g < ng) ws.logits[(long)(hq0 + g) * ws.total_scores + st.score_offsets[b] + j] = x;
+            if (live && j <= row_last[r] && j >= row_first[r]) {
+                x = ws.alibi ? sc[r] + slope[r] * (float)(j - row_last[r]) : sc[r];
+                if (keep_logits) ws.logits[(long)(hq0 + r) * ws.total_scores + st.score_offsets[b] + j] = x;  // (one token: r = head)
             }
-            const float m_new = fmaxf(m[g], wave_max(x));
-            const float corr = (m[g] == -INFINITY) ? 0.0f : __expf(m[g] - m_new);
-            p[g] = live ? __expf(x - m_new) : 0.0f;
-            l[g] = l[g] * corr + wave_sum(p[g]);
+            const float m_new = fmaxf(m[r], wave_max(x));
+            const float corr = (m[r] == -INFINITY) ? 0.0f : __expf(m[r] - m_new);
+            p[r] = x == -INFINITY ? 0.0f : __expf(x - m_new);  // (a row that has seen nothing yet: m_new = -inf too)
+            l[r] = l[r] * corr + wave_sum(p[r]);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[g][e] *= corr;
-            zacc[g] *= corr;
-            m[g] = m_new;
+            for (int e = 0; e < 8; ++e) acc[r][e] *= corr;
+            zacc[r] *= corr;
+            m[r] = m_new;
         }
         const int cnt = min(64, j_end - j0);
-        for (int r = 0; r * rps < cnt; ++r) {
-            const int jj = r * rps + vrow;            // the row of this lane's group in this step
+        for (int s = 0; s * rps < cnt; ++s) {
+            const int jj = s * rps + vrow;            // the row of this lane's group in this step
             const int src = min(jj, 63);
             const long pb = __shfl(phys, src, WAVE);
             float pj[GC];
 #pragma unroll
-            for (int g = 0; g < GC; ++g) pj[g] = __shfl(p[g], src, WAVE);
+            for (int r = 0; r < GC; ++r) pj[r] = __shfl(p[r], src, WAVE);
             if (v_active && jj < cnt) {
                 RowReader vr(value_cache, pb, hkv, (j0 + jj) % sh.bs, sh.Hkv, sh.bs, Dv, sh.vdt);
                 float v8[8];
                 vr.load8_codes(8 * vlane, v8);
 #pragma unroll
-                for (int g = 0; g < GC; ++g) {
-                    const float w = pj[g] * vr.scale;
-                    zacc[g] += w * vr.zp;
+                for (int r = 0; r < GC; ++r) {
+                    const float w = pj[r] * vr.scale;
+                    zacc[r] += w * vr.zp;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[g][e] += w * v8[e];
+                    for (int e = 0; e < 8; ++e) acc[r][e] += w * v8[e];
                 }
             }
         }
     }
     // the zero-point terms of the lane's rows, then the row groups' partial sums: lanes with the same channels add up
 #pragma unroll
-    for (int g = 0; g < GC; ++g)
+    for (int r = 0; r < GC; ++r)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            acc[g][e] -= zacc[g];
-            for (int o = lpr; o < 64; o <<= 1) acc[g][e] += __shfl_xor(acc[g][e], o, WAVE);
+            acc[r][e] -= zacc[r];
+            for (int o = lpr; o < 64; o <<= 1) acc[r][e] += __shfl_xor(acc[r][e], o, WAVE);
         }
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-        if (g >= ng) break;
-        const long slot = ((long)t * sh.Hq + hq0 + g) * ws.nsplit + split;
+    for (int r = 0; r < GC; ++r) {
+        if (row_last[r] < 0) continue;
+        const int ti = r / hs, g = r - ti * hs;
+        const long slot = ((long)(t0 + ti) * sh.Hq + hq0 + g) * ws.nsplit + split;
         if (lane == 0) {
-            ws.part_ml[2 * slot] = m[g];
-            ws.part_ml[2 * slot + 1] = l[g];
+            ws.part_ml[2 * slot] = m[r];
+            ws.part_ml[2 * slot + 1] = l[r];
         }
         if (vrow == 0 && v_active) {
             float* dst = ws.part_acc + slot * Dv + 8 * vlane;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dst[e] = acc[g][e];
+            for (int e = 0; e < 8; ++e) dst[e] = acc[r][e];
         }
     }
 }
@@ -440,8 +456,9 @@ template <int QDT>
 hipError_t launch_typed(hipStream_t s, const StepDev& st, const GenericShape& sh, const void* query, const void* kc,
                         const void* vc, const int32_t* bi, const AttnWorkspace& ws, void* out, float* scores,
                         int32_t max_kv_len, hipEvent_t ev0, hipEvent_t ev1) {
-    const int gc = generic_heads_per_wave(sh);
-    const long waves = (long)st.T * sh.Hkv * ceil_div(sh.Hq / sh.Hkv, gc) * ws.nsplit;
+    const GenericPlan plan = generic_plan(sh, st.T > st.B);
+    const int gc = plan.rows, hs = plan.heads;
+    const long waves = (long)st.n_gtiles * sh.Hkv * ceil_div(sh.Hq / sh.Hkv, hs) * ws.nsplit;
     if (waves == 0) return hipSuccess;
     auto q = reinterpret_cast<const uint16_t*>(query);
     auto k = reinterpret_cast<const uint8_t*>(kc);
@@ -450,10 +467,10 @@ hipError_t launch_typed(hipStream_t s, const StepDev& st, const GenericShape& sh
     const size_t lds = (size_t)4 * gc * sh.Dk * sizeof(float);
     if (ev0) (void)hipEventRecord(ev0, s);
     switch (gc) {
-        case 1: hipLaunchKernelGGL((pa_generic_kernel<QDT, 1>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
-        case 2: hipLaunchKernelGGL((pa_generic_kernel<QDT, 2>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
-        case 4: hipLaunchKernelGGL((pa_generic_kernel<QDT, 4>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
-        default: hipLaunchKernelGGL((pa_generic_kernel<QDT, 8>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0); break;
+        case 1: hipLaunchKernelGGL((pa_generic_kernel<QDT, 1>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0, hs); break;
+        case 2: hipLaunchKernelGGL((pa_generic_kernel<QDT, 2>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0, hs); break;
+        case 4: hipLaunchKernelGGL((pa_generic_kernel<QDT, 4>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0, hs); break;
+        default: hipLaunchKernelGGL((pa_generic_kernel<QDT, 8>), grid, block, lds, s, st, sh, q, k, v, bi, ws, scores ? 1 : 0, hs); break;
     }
     if (ev1) (void)hipEventRecord(ev1, s);
     const long rows = (long)st.T * sh.Hq;

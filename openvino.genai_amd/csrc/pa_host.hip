@@ -1078,8 +1078,10 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         PA_REQUIRE((int64_t)T * ctx->cfg.num_heads <= INT32_MAX, PA_OUT_OF_BOUNDS,
                    "tokens x query heads of a step overflow int32");
 
-        // pack the device copy: past | sb | bib | window | score_off | token_seq
-        std::vector<int32_t> h((size_t)B + (B + 1) + (B + 1) + B + (B + 1) + T);
+        // pack the device copy: past | sb | bib | window | score_off | token_seq | token tiles of the generic kernel
+        const pa::GenericShape gsh = generic_shape_of(ctx->cfg);
+        const pa::GenericPlan gplan = pa::generic_plan(gsh, T > B);
+        std::vector<int32_t> h((size_t)B + (B + 1) + (B + 1) + B + (B + 1) + T + T);
         int32_t* past = h.data();
         int32_t* sb = past + B;
         int32_t* bib = sb + B + 1;
@@ -1098,6 +1100,13 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
             soff[b + 1] = soff[b] + past[b] + q_len;
             for (int32_t t = sb[b]; t < sb[b + 1]; ++t) tseq[t] = b;
         }
+        PA_REQUIRE((int64_t)T * 8 <= INT32_MAX, PA_OUT_OF_BOUNDS, "too many tokens in a step");
+        int32_t* gtiles = tseq + T;
+        int32_t n_gtiles = 0;
+        for (int32_t b = 0; b < B; ++b)
+            for (int32_t t = sb[b]; t < sb[b + 1]; t += gplan.tokens)
+                gtiles[n_gtiles++] = t * 8 + (std::min(gplan.tokens, sb[b + 1] - t) - 1);
+
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         // the previous step's kernels may still read the old copy
         HIP_CHECK(hipStreamSynchronize(ctx->stream));
@@ -1112,6 +1121,8 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         ctx->dev.score_window = d + B + 2 * (B + 1);
         ctx->dev.score_offsets = d + 2 * B + 2 * (B + 1);
         ctx->dev.token_seq = d + 2 * B + 3 * (B + 1);
+        ctx->dev.gtiles = ctx->dev.token_seq + T;
+        ctx->dev.n_gtiles = n_gtiles;
         ctx->dev.B = B;
         ctx->dev.T = T;
         ctx->dev.sliding_window = m->sliding_window;
@@ -1127,10 +1138,8 @@ int32_t pa_step_begin(pa_ctx* ctx, const pa_step_meta* m) {
         ctx->h_sb.assign(sb, sb + B + 1);
         ctx->h_bib.assign(bib, bib + B + 1);
         // split-K plan: enough waves to fill 256 CUs several times over, at least 256 positions per split
-        // (a wave of the shape-generic kernel serves up to eight heads of a kv head's group)
-        const pa::GenericShape gsh = generic_shape_of(ctx->cfg);
-        const int gc = pa::generic_heads_per_wave(gsh);
-        const int64_t rows = (int64_t)T * gsh.Hkv * pa::ceil_div(gsh.Hq / gsh.Hkv, gc);
+        // (a wave of the shape-generic kernel serves a token tile's rows of up to eight heads of a kv head's group)
+        const int64_t rows = std::max<int64_t>(1, (int64_t)n_gtiles * gsh.Hkv * pa::ceil_div(gsh.Hq / gsh.Hkv, gplan.heads));
         const int32_t eff_kv = m->sliding_window > 0 ? std::min(max_kv, m->sliding_window) : max_kv;
         int64_t want = (4096 + rows - 1) / rows;
         int64_t cap = std::max<int64_t>(1, eff_kv / 256);

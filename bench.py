@@ -31,7 +31,7 @@ MEASURED_TRAFFIC = {
     "llama3_8b_decode_u8_b64_ctx4096": (585.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
     "llama3_8b_eviction_u8_b256_ctx8192": (4656.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_eviction_u8_b256_ctx8192.md"),
     "long_context_decode_u8_b8_ctx32768": (594.4e6, "profiles/pa_decode_u8_kernel__long_context_decode_u8_b8_ctx32768.md"),
-    "qwen25_7b_mixed_bf16": (843.1e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
+    "qwen25_7b_mixed_bf16": (218.8e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
 }
 
 

@@ -149,7 +149,8 @@ typedef struct pa_layer_io {
  * value precision of its own, u4 rows, a 16-bit cache of the other 16-bit type, other block sizes) runs on shape-generic
  * kernels, correct but far from the tuned ones' speed.  In a step whose sequences all schedule one token, over a cache
  * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
- * writes). */
+ * writes).  Head size 96 (K and V alike, the same caches): steps with a multi-token sequence run on the tuned matrix
+ * kernel, steps of single-token sequences alone and the append on the shape-generic kernels. */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The op's `alibi_slopes` input (input 11: f32 [num_heads]; a graph constant that SDPAToPagedAttention leaves empty
  * for models without ALiBi, and that the reference never sets itself): with slopes set, every logit gets

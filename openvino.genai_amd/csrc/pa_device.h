@@ -449,7 +449,7 @@ __device__ __forceinline__ float2 row_max_and_sum(const float* __restrict__ fina
     return fold_max_and_sum(reinterpret_cast<const float2*>(m.part_ml) + rid * m.max_split, ns);
 }
 
-// Sixteen lanes per row, D / 16 channels each (16-byte loads), four rows per wave, workgroup `wg` of 256 threads;
+// Sixteen lanes per row, D / 16 channels each (16-byte loads; 8-byte ones when D / 16 is not a multiple of 4), four rows per wave, workgroup `wg` of 256 threads;
 // ranges are folded in ascending order.  DT: type of the output rows.
 template <int D, int DT>
 __device__ __forceinline__ void merge_rows(const MergeRows& a, long wg) {
@@ -485,21 +485,32 @@ __device__ __forceinline__ void merge_rows(const MergeRows& a, long wg) {
         // a round's loads are in flight together
         for (int s0 = 0; s0 < ns; s0 += 4) {
             float f[4];
-            f4_ v[4][EPL / 4];
+            float v[4][EPL];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const long slot = row * a.max_split + min(s0 + j, ns - 1);
                 f[j] = __shfl(f_mine, min(s0 + j, ns - 1), 16);
                 if (s0 + j >= ns) f[j] = 0.0f;
-                const f4_* pa = reinterpret_cast<const f4_*>(a.part_acc + slot * D + l16 * EPL);
+                const float* pa = a.part_acc + slot * D + l16 * EPL;
+                if constexpr (EPL % 4 == 0) {
 #pragma unroll
-                for (int e = 0; e < EPL / 4; ++e) v[j][e] = pa[e];
+                    for (int e = 0; e < EPL / 4; ++e) {
+                        const f4_ x = reinterpret_cast<const f4_*>(pa)[e];
+                        v[j][4 * e] = x[0], v[j][4 * e + 1] = x[1], v[j][4 * e + 2] = x[2], v[j][4 * e + 3] = x[3];
+                    }
+                } else {  // (a lane's channels start on an 8-byte boundary only)
+#pragma unroll
+                    for (int e = 0; e < EPL / 2; ++e) {
+                        const float2 x = reinterpret_cast<const float2*>(pa)[e];
+                        v[j][2 * e] = x.x, v[j][2 * e + 1] = x.y;
+                    }
+                }
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int e = 0; e < EPL; ++e)
-                    acc[e] = fmaf(f[j] == 0.0f ? 0.0f : v[j][e / 4][e % 4], f[j], acc[e]);  // fully masked ranges hold nothing
+                    acc[e] = fmaf(f[j] == 0.0f ? 0.0f : v[j][e], f[j], acc[e]);  // fully masked ranges hold nothing
         }
     } else {
         M = -INFINITY;
@@ -523,7 +534,11 @@ __device__ __forceinline__ void merge_rows(const MergeRows& a, long wg) {
         o[e] = (uint32_t)store16<DT>(acc[2 * e] * inv) | ((uint32_t)store16<DT>(acc[2 * e + 1] * inv) << 16);
     uint16_t* dst = a.out + row * D + l16 * EPL;
     if constexpr (EPL == 8) *reinterpret_cast<u4_*>(dst) = u4_{o[0], o[1], o[2], o[3]};
-    else *reinterpret_cast<uint2*>(dst) = make_uint2(o[0], o[1]);
+    else if constexpr (EPL == 4) *reinterpret_cast<uint2*>(dst) = make_uint2(o[0], o[1]);
+    else {
+#pragma unroll
+        for (int e = 0; e < EPL / 2; ++e) reinterpret_cast<uint32_t*>(dst)[e] = o[e];
+    }
     if (l16 == 0) {
         a.final_ml[2 * row] = M * LN2_;
         a.final_ml[2 * row + 1] = L;

@@ -972,7 +972,7 @@ template <int D, int DT, int QDT, bool U8>
 static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1,
                                          bool merge_later) {
     if (ev0) (void)hipEventRecord(ev0, s);
-    if constexpr (U8) {
+    if constexpr (U8 && D != 96) {
         if (a.n_wide > 0) {  // u8 caches: the items with more than 16 query rows (up to 128) come first in the list
             PrefillArgs w = a;
             w.n_items = a.n_wide;
@@ -1030,6 +1030,7 @@ hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, in
     if (a.n_items == 0) return hipSuccess;
     if (a.sh.D == 128) return launch_prefill16_d<128>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     if (a.sh.D == 64) return launch_prefill16_d<64>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
+    if (a.sh.D == 96) return launch_prefill16_d<96>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     return hipErrorInvalidValue;
 }
 

@@ -15,6 +15,9 @@ MIXES = [
     ("bf16", 256, 256, "bf16", "bf16", 32, 4, 1), ("f16", 128, 64, "u8", "f16", 32, 8, 2), ("bf16", 64, 128, "bf16", "u8", 32, 8, 2),
     ("f16", 192, 128, "f16", "u4", 32, 6, 3), ("bf16", 128, 128, "u4", "u4", 32, 8, 2), ("f16", 72, 40, "u4", "bf16", 24, 4, 2),
     ("f16", 128, 128, "bf16", "bf16", 32, 8, 2), ("f16", 512, 8, "u8", "u8", 32, 2, 1),
+    # head size 96 (K and V alike, a u8 cache or one of the query's type): the matrix kernel's one-row-group variants
+    ("f16", 96, 96, "f16", "f16", 32, 8, 8), ("bf16", 96, 96, "bf16", "bf16", 32, 6, 2), ("f16", 96, 96, "u8", "u8", 32, 12, 4),
+    ("bf16", 96, 96, "u8", "u8", 64, 4, 1),
 ]
 
 

@@ -103,7 +103,9 @@ __device__ __forceinline__ void issue_block(const DecodeArgs& a, int phys0, int 
 }
 
 template <int D, int QDT, int WAVES, int BS>
-__global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs a) {
+// (head size 256: one workgroup per CU, whose waves may then use the accumulation registers as well -- 16 KB blocks,
+// two of them in flight, 64 accumulators and 32 query registers do not fit 256 registers)
+__global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 2) void pa_decode_u8_kernel(DecodeArgs a) {
     constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile
     static_assert(BS == 32 || (BS == 16 && WAVES == 4), "the descriptor holds the ids of the first eight tiles");
     // BS = 32 stands for every block size from 32 tokens up (a power of two): a tile is then one 32-token part of a
@@ -118,8 +120,17 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     constexpr int KS = D / 32;             // k-steps of the QK contraction
     constexpr int RT = D / 16;             // 16-row output tiles of PV
     constexpr int VB = D / 16;             // V bytes per lane per token row
+    constexpr int NW = (VB + 3) / 4;       // ... held in this many 32-bit words
     constexpr int SLOT = TILE;             // a wave's LDS staging slot: a K block, then a V block
-    constexpr int EPL = D / 64;            // elements per lane of a new K / V row
+    constexpr int EPL = (D + 63) / 64;     // elements per lane of a new K / V row
+    constexpr bool CAN_APPEND = D % 64 == 0;  // (a row of the fused append is spread over all 64 lanes)
+    constexpr int DEPTH = 2;               // blocks a wave keeps in flight
+    // Channel of row m of output tile r (the lane with n = m reads that channel's byte of each of its token rows): a
+    // lane's VB consecutive channels, except that with 6 bytes per lane (D = 96) the lanes take four consecutive
+    // channels of the first 64 and two of the last 32, so that their reads stay aligned.
+    auto chan = [](const int m, const int r) __attribute__((always_inline)) {
+        return D == 96 ? (r < 4 ? 4 * m + r : 64 + 2 * m + (r - 4)) : VB * m + r;
+    };
     static_assert(TILE == FULL * 1024 + 256, "tile = whole passes + 16 chunks");
     extern __shared__ __align__(16) uint8_t smem[];
 
@@ -150,16 +161,18 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     // see the row, and loads and stores of a wave may complete out of order with respect to each other, so the wave
     // waits for its stores explicitly (vmcnt(0)) before it issues the fetch of that block: at once when the block is
     // among its first ones, else (the stores then follow its first fetches) right in front of that fetch.
-    const bool appends = a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
+    const bool appends = CAN_APPEND && a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
     const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
     auto append_rows = [&]() __attribute__((always_inline)) {
-        const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
-        const long dst = (((long)dsc->last_id * Hkv + hkv) * bsz + (kv_len - 1) % bsz) * ROW;
-        uint16_t kr[EPL], vr[EPL];
-        load_row16<EPL>(a.key + src, kr);
-        load_row16<EPL>(a.value + src, vr);
-        quantize_row_u8<QDT, EPL>(kr, const_cast<uint8_t*>(a.key_cache) + dst, lane);
-        quantize_row_u8<QDT, EPL>(vr, const_cast<uint8_t*>(a.value_cache) + dst, lane);
+        if constexpr (CAN_APPEND) {
+            const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
+            const long dst = (((long)dsc->last_id * Hkv + hkv) * bsz + (kv_len - 1) % bsz) * ROW;
+            uint16_t kr[EPL], vr[EPL];
+            load_row16<EPL>(a.key + src, kr);
+            load_row16<EPL>(a.value + src, vr);
+            quantize_row_u8<QDT, EPL>(kr, const_cast<uint8_t*>(a.key_cache) + dst, lane);
+            quantize_row_u8<QDT, EPL>(vr, const_cast<uint8_t*>(a.value_cache) + dst, lane);
+        }
     };
     if (append_first) {
         append_rows();
@@ -171,7 +184,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     int tile = tb + wv;
     if (tile < te)
         issue_block<FULL, BS>(a, dsc->ids[BPT * wv], dsc->ids[BPT * wv + BPT - 1], tile & sub_mask, hkv, TILE, lane, kraw, vraw, traw);
-    if (tile + WAVES < te)
+    if (DEPTH == 2 && tile + WAVES < te)
         issue_block<FULL, BS>(a, dsc->ids[BPT * (wv + WAVES)], dsc->ids[BPT * (wv + WAVES) + BPT - 1], (tile + WAVES) & sub_mask,
                               hkv, TILE, lane, kraw2, vraw2, traw2);
     const bool append_late = appends && !append_first;
@@ -256,10 +269,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
 #pragma unroll
         for (int c = 0; c < FULL; ++c) reinterpret_cast<u4v*>(slot)[c * 64 + lane] = vr[c];
         if (lane >= 16 && lane < 32) reinterpret_cast<u4v*>(slot)[FULL * 64 + lane - 16] = tr;
-        if (append_late && tile + 2 * WAVES == tile_hi - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the appended row is in place
-        if (tile + 2 * WAVES < te) {
-            const int ti = BPT * (tile + 2 * WAVES - tb);
-            issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], (tile + 2 * WAVES) & sub_mask, hkv, TILE, lane, kr, vr, tr);
+        if (append_late && tile + DEPTH * WAVES == tile_hi - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the appended row is in place
+        if (tile + DEPTH * WAVES < te) {
+            const int ti = BPT * (tile + DEPTH * WAVES - tb);
+            issue_block<FULL, BS>(a, tab[ti], tab[ti + BPT - 1], (tile + DEPTH * WAVES) & sub_mask, hkv, TILE, lane, kr, vr, tr);
         }
         __builtin_amdgcn_wave_barrier();
 
@@ -336,18 +349,23 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
         else softmax(std::false_type{});
 
         // ---- O^T[d][head] += V^T . P^T ----------------------------------------------------------
-        // lane (m = n, g) reads its VB bytes d = VB*m .. of each of its eight token rows
-        uint32_t vlo[8], vhi[8];
+        // lane (m = n, g) reads the bytes of its channels chan(m, 0 .. VB - 1) of each of its eight token rows
+        uint32_t vw[NW][8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const uint8_t* p = slot + ROW * (16 * (j >> 2) + 4 * g + (j & 3)) + 8 + VB * n;
-            if (VB == 8) {
-                const uint2 w = *reinterpret_cast<const uint2*>(p);
-                vlo[j] = w.x;
-                vhi[j] = w.y;
+            const uint8_t* p = slot + ROW * (16 * (j >> 2) + 4 * g + (j & 3)) + 8;
+            if constexpr (VB == 16) {  // (rows start on 8-byte boundaries)
+                const uint2 w0 = *reinterpret_cast<const uint2*>(p + 16 * n);
+                const uint2 w1 = *reinterpret_cast<const uint2*>(p + 16 * n + 8);
+                vw[0][j] = w0.x, vw[1][j] = w0.y, vw[2][j] = w1.x, vw[3][j] = w1.y;
+            } else if constexpr (VB == 8) {
+                const uint2 w = *reinterpret_cast<const uint2*>(p + 8 * n);
+                vw[0][j] = w.x, vw[1][j] = w.y;
+            } else if constexpr (VB == 6) {
+                vw[0][j] = *reinterpret_cast<const uint32_t*>(p + 4 * n);
+                vw[1][j] = *reinterpret_cast<const uint16_t*>(p + 64 + 2 * n);
             } else {
-                vlo[j] = *reinterpret_cast<const uint32_t*>(p);
-                vhi[j] = 0;
+                vw[0][j] = *reinterpret_cast<const uint32_t*>(p + 4 * n);
             }
         }
 #pragma unroll
@@ -355,16 +373,15 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
             const uint32_t sel = 0x0c000c00u | (uint32_t)(r & 3) | ((uint32_t)(4 + (r & 3)) << 16);
             u4v av;
 #pragma unroll
-            for (int p = 0; p < 4; ++p)
-                av[p] = (r < 4) ? perm(vlo[2 * p + 1], vlo[2 * p], sel) : perm(vhi[2 * p + 1], vhi[2 * p], sel);
+            for (int p = 0; p < 4; ++p) av[p] = perm(vw[r >> 2][2 * p + 1], vw[r >> 2][2 * p], sel);
             acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), pb, acc[r], 0, 0, 0);
             acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), pl, acc[r], 0, 0, 0);
         }
         __builtin_amdgcn_wave_barrier();
     };
-    for (; tile < te; tile += 2 * WAVES) {
+    for (; tile < te; tile += DEPTH * WAVES) {
         process(kraw, vraw, traw, tile);
-        if (tile + WAVES < te) process(kraw2, vraw2, traw2, tile + WAVES);
+        if (DEPTH == 2 && tile + WAVES < te) process(kraw2, vraw2, traw2, tile + WAVES);
     }
 
     // ---- merge the waves ---------------------------------------------------------------------------
@@ -401,11 +418,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void pa_decode_u8_kernel(DecodeArgs 
     for (int n0 = 0; n0 < G; n0 += HC) {
         if (n0) __syncthreads();
         if (n >= n0 && n < min(G, n0 + HC)) {
-            float* dst = red + ((wv * HC + n - n0) * D) + (D / 4) * g;
+            float* dst = red + ((wv * HC + n - n0) * D);
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) dst[VB * i + r] = acc[r][i];  // lane (n, g), register i of tile r: d = (D/4) g + VB i + r
+                for (int i = 0; i < 4; ++i) dst[chan(4 * g + i, r)] = acc[r][i];  // lane (n, g), register i of tile r: row 4 g + i
         }
         __syncthreads();
         if (n0 == 0 && a.want_scores) {
@@ -507,7 +524,9 @@ __host__ __device__ inline long decode_merge_rows(const DecodeArgs& a) {
 // WRITE_FAC: leave exp2(m_split - M) / L in place of the split denominators (for a score kernel that runs afterwards).
 template <int D, int QDT, bool WRITE_FAC>
 __device__ __forceinline__ void merge_row(const DecodeArgs& a, const long r, const int lane) {
-    constexpr int EPL = D / 64;
+    constexpr int EPL = (D + 63) / 64;  // (D = 96: two channels on each of the first 48 lanes)
+    const bool act = lane * EPL < D;
+    const int ch = act ? lane * EPL : 0;
     if (r >= decode_merge_rows(a)) return;
     long row = r;
     if (a.seq_list) {  // mixed step: the rows of the listed single-token sequences (the others are another kernel's)
@@ -535,7 +554,7 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, const long r, con
             for (int j = 0; j < 8; ++j) {
                 const long slot = row * a.nsplit + min(s0 + j, a.nsplit - 1);
                 ms[j] = a.part_ml[2 * slot];  // same address in every lane: one broadcast load
-                const float* pa = a.part_acc + slot * D + lane * EPL;
+                const float* pa = a.part_acc + slot * D + ch;
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) v[j][e] = pa[e];
             }
@@ -560,7 +579,7 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, const long r, con
             const float f = __builtin_amdgcn_exp2f(ms - M);
             L += a.part_ml[2 * slot + 1] * f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + lane * EPL + e] * f;
+            for (int e = 0; e < EPL; ++e) acc[e] += a.part_acc[slot * D + ch + e] * f;
         }
         inv = L > 0.0f ? 1.0f / L : 0.0f;
         for (int s = lane; WRITE_FAC && s < a.nsplit; s += WAVE) {
@@ -570,7 +589,8 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, const long r, con
         }
     }
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) a.out[row * D + lane * EPL + e] = store16<QDT>(acc[e] * inv);
+    for (int e = 0; e < EPL; ++e)
+        if (act) a.out[row * D + ch + e] = store16<QDT>(acc[e] * inv);
     if (lane == 0) {
         a.final_ml[2 * row] = M;
         a.final_ml[2 * row + 1] = L;
@@ -718,7 +738,11 @@ static hipError_t launch_decode_waves(hipStream_t s, const DecodeArgs& a, float*
         return launch_decode_typed<D, QDT, 4, 16>(s, a, scores, max_kv_len, ev0, ev1);
     }
     if (a.sh.bs < 32 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1))) return hipErrorInvalidValue;
-    if (a.waves == 8) return launch_decode_typed<D, QDT, 8, 32>(s, a, scores, max_kv_len, ev0, ev1);
+    if (a.waves == 8) {
+        // (eight-wave workgroups leave a wave 128 registers: head sizes 64 and 128)
+        if constexpr (D == 64 || D == 128) return launch_decode_typed<D, QDT, 8, 32>(s, a, scores, max_kv_len, ev0, ev1);
+        else return hipErrorInvalidValue;
+    }
     return launch_decode_typed<D, QDT, 4, 32>(s, a, scores, max_kv_len, ev0, ev1);
 }
 
@@ -731,16 +755,18 @@ hipError_t launch_decode_scores(hipStream_t s, const DecodeArgs& a, float* score
 
 hipError_t launch_decode_merge(hipStream_t s, const DecodeArgs& a, int q_dtype) {
     const dim3 grid((unsigned)((decode_merge_rows(a) + 3) / 4));
-    if (a.sh.D == 128) {
-        if (q_dtype == DT_F16) hipLaunchKernelGGL((pa_decode_merge_kernel<128, DT_F16>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((pa_decode_merge_kernel<128, DT_BF16>), grid, dim3(256), 0, s, a);
-    } else if (a.sh.D == 64) {
-        if (q_dtype == DT_F16) hipLaunchKernelGGL((pa_decode_merge_kernel<64, DT_F16>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((pa_decode_merge_kernel<64, DT_BF16>), grid, dim3(256), 0, s, a);
-    } else {
-        return hipErrorInvalidValue;
+#define PA_MERGE(D_)                                                                                              \
+    if (a.sh.D == D_) {                                                                                           \
+        if (q_dtype == DT_F16) hipLaunchKernelGGL((pa_decode_merge_kernel<D_, DT_F16>), grid, dim3(256), 0, s, a); \
+        else hipLaunchKernelGGL((pa_decode_merge_kernel<D_, DT_BF16>), grid, dim3(256), 0, s, a);                  \
+        return hipGetLastError();                                                                                 \
     }
-    return hipGetLastError();
+    PA_MERGE(128)
+    PA_MERGE(64)
+    PA_MERGE(96)
+    PA_MERGE(256)
+#undef PA_MERGE
+    return hipErrorInvalidValue;
 }
 
 template <int D, int QDT>
@@ -756,12 +782,16 @@ static hipError_t launch_post_typed(hipStream_t s, const DecodeArgs& a, float* s
 // What follows a decode launch: with several splits the merge, with scores the score kernel, both in one launch when
 // the factors of a sequence's heads fit a small LDS table.
 hipError_t launch_decode_post(hipStream_t s, const DecodeArgs& a, int q_dtype, float* scores, int max_kv_len) {
-    if (a.nsplit > 1 && scores && a.sh.Hq * a.nsplit <= 4096 && (a.sh.D == 128 || a.sh.D == 64)) {
-        if (a.sh.D == 128)
-            return q_dtype == DT_F16 ? launch_post_typed<128, DT_F16>(s, a, scores, max_kv_len)
-                                     : launch_post_typed<128, DT_BF16>(s, a, scores, max_kv_len);
-        return q_dtype == DT_F16 ? launch_post_typed<64, DT_F16>(s, a, scores, max_kv_len)
-                                 : launch_post_typed<64, DT_BF16>(s, a, scores, max_kv_len);
+    if (a.nsplit > 1 && scores && a.sh.Hq * a.nsplit <= 4096) {
+#define PA_POST(D_)                                                                               \
+    if (a.sh.D == D_)                                                                             \
+        return q_dtype == DT_F16 ? launch_post_typed<D_, DT_F16>(s, a, scores, max_kv_len)       \
+                                 : launch_post_typed<D_, DT_BF16>(s, a, scores, max_kv_len);
+        PA_POST(128)
+        PA_POST(64)
+        PA_POST(96)
+        PA_POST(256)
+#undef PA_POST
     }
     hipError_t e;
     if (a.nsplit > 1 && (e = launch_decode_merge(s, a, q_dtype)) != hipSuccess) return e;
@@ -776,6 +806,12 @@ hipError_t launch_decode_u8(hipStream_t s, const DecodeArgs& a, int q_dtype, flo
     if (a.sh.D == 64)
         return q_dtype == DT_F16 ? launch_decode_waves<64, DT_F16>(s, a, scores, max_kv_len, ev0, ev1)
                                  : launch_decode_waves<64, DT_BF16>(s, a, scores, max_kv_len, ev0, ev1);
+    if (a.sh.D == 96)
+        return q_dtype == DT_F16 ? launch_decode_waves<96, DT_F16>(s, a, scores, max_kv_len, ev0, ev1)
+                                 : launch_decode_waves<96, DT_BF16>(s, a, scores, max_kv_len, ev0, ev1);
+    if (a.sh.D == 256)
+        return q_dtype == DT_F16 ? launch_decode_waves<256, DT_F16>(s, a, scores, max_kv_len, ev0, ev1)
+                                 : launch_decode_waves<256, DT_BF16>(s, a, scores, max_kv_len, ev0, ev1);
     return hipErrorInvalidValue;
 }
 

@@ -346,10 +346,14 @@ void do_kv_append(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
 bool tuned_block_size(int32_t bs) { return bs >= 16 && bs <= 256 && (bs & (bs - 1)) == 0; }
 
 // Shapes the tuned u8 decode kernel is built for (it takes the single-token sequences of a step).
+// (head size 256 with 16-token blocks would spill registers and is left to the shape-generic kernel)
 bool decode_u8_shape(const pa_config& c) {
     return kv_alike(c) && c.kv_cache_dtype == PA_U8 && tuned_block_size(c.block_size) &&
-           (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
+           (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || (c.head_size == 256 && c.block_size >= 32)) &&
+           c.num_heads / c.num_kv_heads <= 16;
 }
+// ... and whose rows the decode kernels can append themselves (a row spread over all 64 lanes).
+bool fused_append_shape(const pa_config& c) { return c.head_size % 64 == 0; }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
@@ -376,6 +380,11 @@ bool decode16_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode16_shap
 // against 1.15); with a multi-token sequence in the step the matrix kernel takes all of it.
 bool matrix_step(const pa_ctx* ctx) {
     return mfma_shape(ctx) && ctx->n_items > 0 && !(ctx->cfg.head_size == 96 && ctx->T == ctx->B);
+}
+// Whether the planned step's single-token sequences run on the u8 decode kernel: next to the matrix kernel, which
+// takes the other sequences, or -- a shape only the decode kernel is built for (head size 256) -- when there are no others.
+bool decode_u8_step(const pa_ctx* ctx) {
+    return decode_u8_shape(ctx) && !ctx->h_dec.empty() && (mfma_shape(ctx) || (int32_t)ctx->h_dec.size() == ctx->B);
 }
 
 // Split-K plan of the decode kernels: workgroups per (sequence, kv head) and the most blocks one walks.
@@ -421,14 +430,16 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
             // rule this replaces -- at least one round of workgroups, at least 16 blocks each, rounds 85 % full --
             // batches of 24 to 56 sequences x 8 kv heads run 10 - 26 % faster, because they are not cut at all; full
             // batches and long contexts come out the same within 2 %.)
+            // (head size 256 runs one workgroup per CU; a tile of it is two tiles of head size 128 in bytes, which two
+            // workgroups sharing a CU take t2 for)
             const bool sc = want_scores;
             const double dscale = c.head_size / 128.0;
-            const double t1 = (u8 ? (sc ? 0.316 : 0.276) : (sc ? 0.495 : 0.478)) * dscale;
             const double t2 = (u8 ? (sc ? 0.525 : 0.468) : (sc ? 1.104 : 1.064)) * dscale;
+            const double t1 = slots == 256 ? t2 / 2 : (u8 ? (sc ? 0.316 : 0.276) : (sc ? 0.495 : 0.478)) * dscale;
             const double tile_bytes = 2.0 * 32 * (u8 ? c.head_size + 8 : 2 * c.head_size), bw = sc ? 5.9e6 : 6.97e6;
             const double post_a = u8 ? (sc ? 2.4 : 1.0) : (sc ? 4.2 : 2.8), post_b = u8 ? (sc ? 0.0079 : 0.0066) : (sc ? 0.0050 : 0.0046);
             auto t_tile = [&](int64_t w) {  // per tile, with w workgroups running at once
-                return std::max(w <= slots / 2 ? t1 : t2, (double)w * tile_bytes / bw);
+                return std::max(w <= slots / 2 || slots == 256 ? t1 : t2, (double)w * tile_bytes / bw);
             };
             // Contexts of unequal length: every sequence is cut into the same number of parts, so its workgroups are
             // as much shorter than the longest one's as its context is; the launch then behaves like one of fewer
@@ -471,11 +482,11 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
         return s;
     };
     int32_t cap4 = 0, waves = 4;
-    int32_t s = plan(4, 512, &cap4);
+    int32_t s = plan(4, u8 && c.head_size > 128 ? 256 : 512, &cap4);
     // A context whose probabilities do not fit half a CU's LDS is cut into splits that send every head's
     // probabilities through HBM and add a merge.  With enough (sequence, kv head) pairs to give every CU a workgroup
     // of its own, one workgroup of eight waves per CU (the same waves per CU, the whole LDS) needs fewer of them.
-    if (u8 && c.block_size >= 32 && most > cap4 && pairs >= 256) {
+    if (u8 && c.block_size >= 32 && c.head_size != 96 && c.head_size <= 128 && most > cap4 && pairs >= 256) {
         int32_t cap8 = 0;
         const int32_t s8 = plan(8, 256, &cap8);
         if (s8 < s) {
@@ -777,7 +788,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
     const int32_t* table = table_for(ctx, layer);
     const pa_config& c = ctx->cfg;
     const size_t rows = (size_t)ctx->T * c.num_heads;
-    const bool use_decode = decode_u8_shape(ctx) && !ctx->h_dec.empty();
+    const bool use_decode = decode_u8_step(ctx);
     const bool use_mfma = matrix_step(ctx);
     // 16-bit caches, no dense chunk in the step: the single-token sequences go to their own decode kernel.  (Next to
     // dense chunks they stay work items of the matrix kernel: bandwidth-bound and matrix-bound items share the CUs
@@ -790,7 +801,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
                    PA_NOT_IMPLEMENTED,
                    "pa_attention_static serves steps in which every sequence schedules one token, over a u8 cache or a "
-                   "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64 or 128, K and V alike; at most 16 heads per kv head)");
+                   "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64 or 128, over u8 also 96 and -- from block size 32 -- 256, K and V alike; at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
     // fork: what is launched on the returned stream starts behind what the context's stream holds so far and runs
@@ -1199,7 +1210,7 @@ void shape_tables(pa_ctx* ctx, bool shared) {
 size_t table_upload_bytes(pa_ctx* ctx, int32_t count, size_t* id_bytes, bool* with_descs) {
     *id_bytes = std::max<size_t>(((size_t)count * sizeof(int32_t) + 127) & ~(size_t)127, 128);
     size_t total = *id_bytes;
-    *with_descs = decode_u8_shape(ctx) && !ctx->h_dec.empty();
+    *with_descs = decode_u8_step(ctx);
     if (*with_descs)
         for (int w = 0; w < 2; ++w) {
             ctx->desc_off[w] = total;
@@ -1473,7 +1484,7 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         // a step of single-token sequences that all go to one of the decode kernels: it appends the new rows itself
         const bool fuse = ctx->step_ready &&
-                          ((decode_u8_shape(ctx) && (int32_t)ctx->h_dec.size() == ctx->B) ||
+                          ((decode_u8_shape(ctx) && fused_append_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B) ||
                            (mfma_shape(ctx) && decode16_shape(ctx) && (int32_t)ctx->h_dec16.size() == ctx->B &&
                             ctx->n_sparse == 0 && ctx->n_single == ctx->n_items));
         if (fuse) check_io(ctx, layer, io, true, false);

@@ -216,6 +216,16 @@ def test_edge_shapes(pkg, dev, name, args):
     ("dec_u8_window_unaligned", (8, 2, 128, 32, "f16", "u8", [300, 77], [1, 1]), {"sliding_window": 45}),
     ("dec_u8_w0_mix", (8, 2, 128, 32, "f16", "u8", [300, 77, 500], [1, 1, 1]), {"score_aggregation_window": [1, 0, 1]}),
     ("dec_u8_many_seqs", (32, 8, 128, 32, "f16", "u8", list(range(1, 600, 9)), [1] * 67), {}),
+    # head sizes 96 (six value channels per lane, append by the shape-generic kernel) and 256 (one workgroup per CU)
+    ("dec_u8_d96_mha_multi_split", (6, 6, 96, 32, "f16", "u8", [3000, 2500, 17], [1, 1, 1]), {}),
+    ("dec_u8_d96_g3_bs16_bf16q", (12, 4, 96, 16, "bf16", "u8", [700, 64, 31, 32, 33, 1500], [1] * 6), {}),
+    ("dec_u8_d96_bs128_window", (8, 2, 96, 128, "f16", "u8", [5000, 900, 40], [1, 1, 1]), {"sliding_window": 1000}),
+    ("dec_u8_d96_many_seqs", (32, 32, 96, 32, "f16", "u8", list(range(1, 600, 9)), [1] * 67), {}),
+    ("dec_u8_d256_g2_multi_split", (16, 8, 256, 32, "f16", "u8", [3000, 2500, 17], [1, 1, 1]), {}),
+    ("dec_u8_d256_mha_bf16q_bs64", (4, 4, 256, 64, "bf16", "u8", [700, 64, 31, 32, 33, 1500], [1] * 6), {}),
+    ("dec_u8_d256_g16_window", (16, 1, 256, 32, "f16", "u8", [5000, 900, 40], [1, 1, 1]), {"sliding_window": 1000}),
+    ("dec_u8_d256_w0_mix", (8, 2, 256, 32, "bf16", "u8", [300, 77, 500], [1, 1, 1]), {"score_aggregation_window": [1, 0, 1]}),
+    ("dec_u8_d256_many_seqs", (16, 8, 256, 32, "f16", "u8", list(range(1, 600, 9)), [1] * 67), {}),
 ])
 def test_decode_u8_kernel_shapes(pkg, dev, name, args, kw):
     got, ref, c = _check(pkg, dev, H.case_from_lens(name, *args, **kw), 31, outliers=True)
@@ -263,6 +273,12 @@ def test_prefill16_kernel_shapes(pkg, dev, name, args, kw):
     ("pf_u8_window", (8, 2, 128, 32, "f16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
     ("pf_u8_prefill_only_long", (8, 2, 128, 32, "f16", "u8", [1500], [700]), {"score_aggregation_window": [16]}),
     ("pf_u8_g32_all_on_matrix_kernel", (32, 1, 128, 32, "f16", "u8", [64, 0, 300], [9, 8, 1]), {}),
+    # head size 96: chunks on the matrix kernel's one-row-group variant, single-token sequences on the decode kernel
+    ("pf_u8_d96_mixed", (12, 4, 96, 32, "f16", "u8", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
+    ("pf_u8_d96_mha_bf16q_window", (6, 6, 96, 64, "bf16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
+    # head size 256: a step with a multi-token sequence runs on the shape-generic kernels, single-token ones included
+    ("pf_u8_d256_mixed_generic", (8, 4, 256, 32, "f16", "u8", [0, 700, 40], [50, 1, 1]), {}),
     ("pf_u8_decode_multi_split_beside_prefill", (8, 2, 128, 32, "f16", "u8", [3000, 0, 2500], [1, 40, 1]), {}),
     ("pf_u8_96_heads_ranges", (96, 8, 128, 32, "f16", "u8", [1200, 2500, 60], [200, 1, 1]), {}),
 ])
@@ -460,16 +476,19 @@ LATE_APPEND = [
     ("f16", "u8", 32, 64, (1100, 1300)), ("bf16", "u8", 16, 64, (1100, 1300)), ("f16", "u8", 64, 64, (1100, 1300)),
     ("f16", "u8", 32, 8, (20000, 33000)), ("bf16", "u8", 32, 8, (26000, 33000)),
     ("f16", "f16", 32, 64, (1100, 1300)), ("bf16", "bf16", 16, 64, (1100, 1300)), ("bf16", "bf16", 32, 8, (20000, 33000)),
+    # head size 256 (a seventh field: query heads, kv heads, head size)
+    ("f16", "u8", 32, 64, (1100, 1300), (16, 8, 256)), ("bf16", "u8", 64, 8, (20000, 33000), (16, 8, 256)),
 ]
+LATE_APPEND = [c if len(c) == 6 else c + ((32, 8, 128),) for c in LATE_APPEND]
 
 
-@pytest.mark.parametrize("qd,kd,bs,B,ctx", LATE_APPEND)
-def test_fused_append_row_is_seen_by_the_launch_that_writes_it(pkg, dev, qd, kd, bs, B, ctx):
+@pytest.mark.parametrize("qd,kd,bs,B,ctx,heads", LATE_APPEND)
+def test_fused_append_row_is_seen_by_the_launch_that_writes_it(pkg, dev, qd, kd, bs, B, ctx, heads):
     """The new token dominates the softmax of one head per kv head, so a stale read of its row fails `out` and
     `scores` outright instead of hiding in the tolerance."""
-    Hq, Hkv, D = 32, 8, 128
+    Hq, Hkv, D = heads
     past = np.linspace(ctx[0], ctx[1], B).astype(np.int64) | 1  # odd: the new row is never a block's first
-    case = H.case_from_lens(f"late_append_{qd}_{kd}_bs{bs}_B{B}", Hq, Hkv, D, bs, qd, kd, past, [1] * B)
+    case = H.case_from_lens(f"late_append_{qd}_{kd}_bs{bs}_B{B}_D{D}", Hq, Hkv, D, bs, qd, kd, past, [1] * B)
     print(f"case {case['name']}", flush=True)
     c = H.build_case(case, 4242)
     _plant_dominant_new_rows(c)

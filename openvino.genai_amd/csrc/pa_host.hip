@@ -357,11 +357,13 @@ bool fused_append_shape(const pa_config& c) { return c.head_size % 64 == 0; }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
-// (head size 96: its one-row-group variants only; the decode kernels, the straight-to-LDS variant and the block-sparse
-// estimate are built for 64 and 128)
+// (head sizes 96 and 256: its one-row-group variants only -- at 256 one workgroup per CU, two blocks of LDS slots fill
+// 103 of its 160 KB; the 16-bit decode kernel, the straight-to-LDS variant and the block-sparse estimate are built for
+// 64 and 128)
+bool narrow_only(const pa_config& c) { return c.head_size == 96 || c.head_size == 256; }
 bool mfma_shape(const pa_config& c) {
     return kv_alike(c) && (c.kv_cache_dtype == PA_U8 || c.kv_cache_dtype == c.query_dtype) && tuned_block_size(c.block_size) &&
-           (c.head_size == 64 || c.head_size == 96 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 256;
+           (c.head_size == 64 || c.head_size == 128 || narrow_only(c)) && c.num_heads / c.num_kv_heads <= 256;
 }
 
 // Shapes the 16-bit decode kernel is built for (single-token sequences of a call that asks for no scores).
@@ -374,12 +376,13 @@ bool decode16_shape(const pa_config& c) {
 bool decode_u8_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode_u8_shape(ctx->cfg); }
 bool mfma_shape(const pa_ctx* ctx) { return !ctx->has_alibi && mfma_shape(ctx->cfg); }
 bool decode16_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode16_shape(ctx->cfg); }
-// Whether the planned step runs on the matrix kernel.  Head size 96 has no decode kernel of its own, and a step of
+// Whether the planned step runs on the matrix kernel.  Over 16-bit caches head sizes 96 and 256 have no decode kernel
+// of their own (over u8 caches the decode kernel takes such steps), and a step of
 // single-token sequences alone is faster on the shape-generic kernel, whose waves share a kv head's rows among the
 // group's heads, than in 16-row tiles that hold one group each (64 x 4096 tokens, 32 heads without grouping: 0.88 ms
 // against 1.15); with a multi-token sequence in the step the matrix kernel takes all of it.
 bool matrix_step(const pa_ctx* ctx) {
-    return mfma_shape(ctx) && ctx->n_items > 0 && !(ctx->cfg.head_size == 96 && ctx->T == ctx->B);
+    return mfma_shape(ctx) && ctx->n_items > 0 && !(narrow_only(ctx->cfg) && ctx->T == ctx->B);
 }
 // Whether the planned step's single-token sequences run on the u8 decode kernel: next to the matrix kernel, which
 // takes the other sequences, or -- a shape only the decode kernel is built for (head size 256) -- when there are no others.
@@ -549,7 +552,7 @@ void plan_items(pa_ctx* ctx) {
     // launches to the straight-to-LDS variant).  u8 caches: items with more than 16 rows go to a variant of their own
     // (32 rows per wave, two waves per SIMD) and are listed first
     const bool narrow_all = ctx->cfg.kv_cache_dtype != PA_U8;
-    const bool no_wide = narrow_all || ctx->cfg.head_size == 96;  // (the 32-rows-per-wave u8 variant: head size 64 / 128)
+    const bool no_wide = narrow_all || narrow_only(ctx->cfg);  // (the 32-rows-per-wave u8 variant: head size 64 / 128)
     const int32_t QT = std::max(1, 128 / G), QTX = std::max(1, 128 / G), sw = ctx->sliding_window;
     struct Tile { int32_t b, q0, nq, lo, hi, kind; };  // kind 0: more than 16 rows, 1: the rest, 2: single-token sequences, 3: block-sparse
     std::vector<int32_t> single_idx(B, -1);
@@ -1335,7 +1338,7 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
             return;
         }
         PA_REQUIRE(!ctx->has_alibi, PA_NOT_IMPLEMENTED, "block-sparse prefill is not available with ALiBi slopes");
-        PA_REQUIRE(mfma_shape(c) && c.head_size != 96 && c.block_size >= 32, PA_NOT_IMPLEMENTED,
+        PA_REQUIRE(mfma_shape(c) && !narrow_only(c) && c.block_size >= 32, PA_NOT_IMPLEMENTED,
                    "block-sparse prefill needs a block_size of 32 to 256 (a power of two), head_size 64 or 128 and a u8 cache "
                    "or one of the query's type");
         auto pow2 = [](int32_t v) { return v > 0 && (v & (v - 1)) == 0; };

@@ -184,7 +184,7 @@ __device__ __forceinline__ void wait_vmem() {
 // staging registers the kernel fits three waves per SIMD at two 16-row groups per wave: half the LDS operand traffic
 // per matrix instruction of the one-group variant.
 template <int D, int DT, int QDT, bool U8, int NG, bool XATT, bool DMA, bool HALF = false>
-__global__ __launch_bounds__((DMA || HALF) ? 256 : 512, (DMA || HALF) ? 2 : U8 ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
+__global__ __launch_bounds__((DMA || HALF) ? 256 : 512, D > 128 ? 1 : (DMA || HALF) ? 2 : U8 ? 2 : (XATT && DT == DT_F16 && D == 128) ? 3 : 4)
 void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(!U8 || DT == DT_F16, "u8 codes are multiplied as f16");
     static_assert(U8 || DT == QDT, "16-bit caches are used in the query's type");
@@ -192,7 +192,7 @@ void pa_prefill16_kernel(PrefillArgs a) {
     static_assert(!(DMA && HALF) && (!HALF || (NG == 2 && !XATT)), "the register variant of 256 threads: dense items, two row groups per wave");
     constexpr int NT = (DMA || HALF) ? 256 : 512;
     constexpr int NCH = TOK * (D * 2 / 16);  // 16-byte chunks (eight codes of a u8 row) per block and tensor: 512 (D = 128) or 256 (D = 64)
-    constexpr int UPT = HALF ? NCH / NT : 1;  // load units (a chunk, or eight codes and a row header) per thread and tensor
+    constexpr int UPT = (NCH + NT - 1) / NT;  // load units (a chunk, or eight codes and a row header) per thread and tensor
     constexpr int ROWB = D * 2;            // bytes of a row as staged in LDS
     constexpr int CROWB = U8 ? D + 8 : D * 2;  // bytes of a row in the cache
     constexpr int LROWK = DMA ? ROWB : ROWB + 16;  // LDS row strides chosen so that the operand reads are bank-conflict free:
@@ -972,7 +972,7 @@ template <int D, int DT, int QDT, bool U8>
 static hipError_t launch_prefill16_typed(hipStream_t s, const PrefillArgs& a, hipEvent_t ev0, hipEvent_t ev1,
                                          bool merge_later) {
     if (ev0) (void)hipEventRecord(ev0, s);
-    if constexpr (U8 && D != 96) {
+    if constexpr (U8 && D != 96 && D != 256) {
         if (a.n_wide > 0) {  // u8 caches: the items with more than 16 query rows (up to 128) come first in the list
             PrefillArgs w = a;
             w.n_items = a.n_wide;
@@ -1031,6 +1031,7 @@ hipError_t launch_prefill16(hipStream_t s, const PrefillArgs& a, int q_dtype, in
     if (a.sh.D == 128) return launch_prefill16_d<128>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     if (a.sh.D == 64) return launch_prefill16_d<64>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     if (a.sh.D == 96) return launch_prefill16_d<96>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
+    if (a.sh.D == 256) return launch_prefill16_d<256>(s, a, q_dtype, kv_dtype, ev0, ev1, merge_later);
     return hipErrorInvalidValue;
 }
 

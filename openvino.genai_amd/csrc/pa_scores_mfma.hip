@@ -248,6 +248,8 @@ hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& s
         if (sh.D == 128 && q_dtype == DT_BF16) PA_REPLAY(128, DT_F16, DT_BF16, true)
         if (sh.D == 96 && q_dtype == DT_F16) PA_REPLAY(96, DT_F16, DT_F16, true)
         if (sh.D == 96 && q_dtype == DT_BF16) PA_REPLAY(96, DT_F16, DT_BF16, true)
+        if (sh.D == 256 && q_dtype == DT_F16) PA_REPLAY(256, DT_F16, DT_F16, true)
+        if (sh.D == 256 && q_dtype == DT_BF16) PA_REPLAY(256, DT_F16, DT_BF16, true)
     } else if (kv_dtype == q_dtype) {
         if (sh.D == 64 && q_dtype == DT_F16) PA_REPLAY(64, DT_F16, DT_F16, false)
         if (sh.D == 64 && q_dtype == DT_BF16) PA_REPLAY(64, DT_BF16, DT_BF16, false)
@@ -255,6 +257,8 @@ hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& s
         if (sh.D == 128 && q_dtype == DT_BF16) PA_REPLAY(128, DT_BF16, DT_BF16, false)
         if (sh.D == 96 && q_dtype == DT_F16) PA_REPLAY(96, DT_F16, DT_F16, false)
         if (sh.D == 96 && q_dtype == DT_BF16) PA_REPLAY(96, DT_BF16, DT_BF16, false)
+        if (sh.D == 256 && q_dtype == DT_F16) PA_REPLAY(256, DT_F16, DT_F16, false)
+        if (sh.D == 256 && q_dtype == DT_BF16) PA_REPLAY(256, DT_BF16, DT_BF16, false)
     }
 #undef PA_REPLAY
     return hipErrorInvalidValue;

@@ -260,6 +260,15 @@ def test_decode_u8_kernel_shapes(pkg, dev, name, args, kw):
     ("pf16_bf16_128_heads_ranges", (128, 8, 128, 32, "bf16", "bf16", [1500, 2000, 40], [300, 1, 1]), {}),
     ("pf16_f16_96_heads_ranges_window_rows", (96, 8, 128, 32, "f16", "f16", [1200, 900], [200, 1]),
      {"score_aggregation_window": [5, 1]}),
+    # head sizes 96 and 256 over 16-bit caches: the one-row-group variant (256: one workgroup per CU, two load units
+    # per thread), single-token sequences of a mixed step as its work items
+    ("pf16_bf16_d256_mixed", (16, 8, 256, 32, "bf16", "bf16", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
+    ("pf16_f16_d256_ranges_bs16", (8, 2, 256, 16, "f16", "f16", [3000, 0, 900], [300, 130, 1]), {}),
+    ("pf16_f16_d256_window", (4, 4, 256, 128, "f16", "f16", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
+    ("pf16_bf16_d96_mixed", (12, 4, 96, 32, "bf16", "bf16", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
+     {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
+    ("pf16_f16_d96_ranges_bs64", (6, 6, 96, 64, "f16", "f16", [3000, 0, 900], [300, 130, 1]), {}),
 ])
 def test_prefill16_kernel_shapes(pkg, dev, name, args, kw):
     _check(pkg, dev, H.case_from_lens(name, *args, **kw), 41)
@@ -277,8 +286,11 @@ def test_prefill16_kernel_shapes(pkg, dev, name, args, kw):
     ("pf_u8_d96_mixed", (12, 4, 96, 32, "f16", "u8", [0, 700, 333, 40, 2000, 90], [150, 37, 1, 1, 64, 1]),
      {"score_aggregation_window": [8, 37, 1, 0, 3, 1]}),
     ("pf_u8_d96_mha_bf16q_window", (6, 6, 96, 64, "bf16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
-    # head size 256: a step with a multi-token sequence runs on the shape-generic kernels, single-token ones included
-    ("pf_u8_d256_mixed_generic", (8, 4, 256, 32, "f16", "u8", [0, 700, 40], [50, 1, 1]), {}),
+    # head size 256: chunks on the one-row-group variant with one workgroup per CU
+    ("pf_u8_d256_mixed", (8, 4, 256, 32, "f16", "u8", [0, 700, 40], [50, 1, 1]), {}),
+    ("pf_u8_d256_ranges_window_rows", (16, 8, 256, 64, "bf16", "u8", [3000, 0, 900], [300, 130, 1]),
+     {"score_aggregation_window": [5, 130, 1]}),
+    ("pf_u8_d256_sliding_window", (4, 1, 256, 32, "f16", "u8", [300, 0, 1000], [200, 130, 1]), {"sliding_window": 100}),
     ("pf_u8_decode_multi_split_beside_prefill", (8, 2, 128, 32, "f16", "u8", [3000, 0, 2500], [1, 40, 1]), {}),
     ("pf_u8_96_heads_ranges", (96, 8, 128, 32, "f16", "u8", [1200, 2500, 60], [200, 1, 1]), {}),
 ])

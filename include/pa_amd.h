@@ -149,11 +149,10 @@ typedef struct pa_layer_io {
  * value precision of its own, u4 rows, a 16-bit cache of the other 16-bit type, other block sizes) runs on shape-generic
  * kernels, correct but far from the tuned ones' speed.  In a step whose sequences all schedule one token, over a cache
  * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
- * writes).  Head size 96 (K and V alike, the same caches): sequences that schedule several tokens run on the tuned
- * matrix kernel, single-token sequences over a u8 cache on the tuned decode kernel (over a 16-bit cache: steps of
- * single-token sequences alone on the shape-generic kernel), the append on the shape-generic kernel.  Head size 256
- * over a u8 cache with blocks of 32 tokens or more: steps of single-token sequences alone run on the tuned decode
- * kernel (which appends their rows), every other step on the shape-generic kernels. */
+ * writes).  Head sizes 96 and 256 (K and V alike, the same caches) run on instantiations of the same kernels with
+ * these limits: the matrix kernel keeps to 16 query rows per wave, block-sparse prefill is not offered, the u8 decode
+ * kernel does not take head size 256 with 16-token blocks (such steps run on the shape-generic kernel), and at head
+ * size 96 the append of a step's rows over a u8 cache is always a launch of its own. */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The op's `alibi_slopes` input (input 11: f32 [num_heads]; a graph constant that SDPAToPagedAttention leaves empty
  * for models without ALiBi, and that the reference never sets itself): with slopes set, every logit gets
@@ -171,8 +170,8 @@ int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* pa_attention for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as pa_attention, for steps
  * in which every sequence schedules one token, over a u8 cache or a 16-bit cache of the query's type (block size 16 to
- * 256, a power of two; head size 64 or 128, over u8 also 96 and -- from block size 32 -- 256, K and V alike; at most 16
- * query heads per kv head); other steps return
+ * 256, a power of two; head size 64, 96, 128 or 256 -- over u8 with 16-token blocks not 256 --, K and V alike; at most
+ * 16 query heads per kv head); other steps return
  * PA_NOT_IMPLEMENTED.  The split partials,
  * final maxima / denominators and the score staging live in a fixed device array of PA_STATIC_SCRATCH_BYTES bytes
  * (32 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls

@@ -66,8 +66,10 @@ __device__ __forceinline__ float group_sum(float v) {
     return v + __shfl_xor(v, 32, WAVE);
 }
 
+// (head size 256: one workgroup per CU, whose waves may then use the accumulation registers as well -- two 32 KB
+// blocks in flight are 256 registers by themselves)
 template <int D, int DT, int BS>
-__global__ __launch_bounds__(256, 2) void pa_decode16_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void pa_decode16_kernel(DecodeArgs a) {
     constexpr int WAVES = 4;
     constexpr int BPT = TOK / BS;          // cache blocks per 32-token tile (with two, each holds one row group)
     // BS = 32 stands for every block size from 32 tokens up (a power of two): a tile is then one 32-token part of a block
@@ -431,6 +433,8 @@ hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float*
     hipError_t e;
     if (a.sh.D == 128) e = dtype == DT_F16 ? launch_decode16_typed<128, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<128, DT_BF16>(s, a, ev0, ev1);
     else if (a.sh.D == 64) e = dtype == DT_F16 ? launch_decode16_typed<64, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<64, DT_BF16>(s, a, ev0, ev1);
+    else if (a.sh.D == 96) e = dtype == DT_F16 ? launch_decode16_typed<96, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<96, DT_BF16>(s, a, ev0, ev1);
+    else if (a.sh.D == 256) e = dtype == DT_F16 ? launch_decode16_typed<256, DT_F16>(s, a, ev0, ev1) : launch_decode16_typed<256, DT_BF16>(s, a, ev0, ev1);
     else return hipErrorInvalidValue;
     if (e != hipSuccess) return e;
     return launch_decode_post(s, a, dtype, scores, max_kv_len);

@@ -369,20 +369,22 @@ bool mfma_shape(const pa_config& c) {
 // Shapes the 16-bit decode kernel is built for (single-token sequences of a call that asks for no scores).
 bool decode16_shape(const pa_config& c) {
     return kv_alike(c) && c.kv_cache_dtype != PA_U8 && c.kv_cache_dtype == c.query_dtype && tuned_block_size(c.block_size) &&
-           (c.head_size == 64 || c.head_size == 128) && c.num_heads / c.num_kv_heads <= 16;
+           (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || c.head_size == 256) &&
+           c.num_heads / c.num_kv_heads <= 16;
 }
 
 // The same questions asked of a context: one with ALiBi slopes has no tuned attention kernel.
 bool decode_u8_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode_u8_shape(ctx->cfg); }
 bool mfma_shape(const pa_ctx* ctx) { return !ctx->has_alibi && mfma_shape(ctx->cfg); }
 bool decode16_shape(const pa_ctx* ctx) { return !ctx->has_alibi && decode16_shape(ctx->cfg); }
-// Whether the planned step runs on the matrix kernel.  Over 16-bit caches head sizes 96 and 256 have no decode kernel
-// of their own (over u8 caches the decode kernel takes such steps), and a step of
-// single-token sequences alone is faster on the shape-generic kernel, whose waves share a kv head's rows among the
+// Whether the planned step runs on the matrix kernel (or, a step of single-token sequences over a 16-bit cache, on the
+// 16-bit decode kernel, which is launched in its place).  With more than 16 heads per kv head there is no decode
+// kernel, and at head sizes 96 and 256 a step of
+// single-token sequences alone is then faster on the shape-generic kernel, whose waves share a kv head's rows among the
 // group's heads, than in 16-row tiles that hold one group each (64 x 4096 tokens, 32 heads without grouping: 0.88 ms
 // against 1.15); with a multi-token sequence in the step the matrix kernel takes all of it.
 bool matrix_step(const pa_ctx* ctx) {
-    return mfma_shape(ctx) && ctx->n_items > 0 && !(narrow_only(ctx->cfg) && ctx->T == ctx->B);
+    return mfma_shape(ctx) && ctx->n_items > 0 && !(narrow_only(ctx->cfg) && ctx->T == ctx->B && !decode16_shape(ctx));
 }
 // Whether the planned step's single-token sequences run on the u8 decode kernel: next to the matrix kernel, which
 // takes the other sequences, or -- a shape only the decode kernel is built for (head size 256) -- when there are no others.
@@ -485,7 +487,7 @@ void plan_decode_u8(const pa_ctx* ctx, bool want_scores, int32_t* nsplit_out, in
         return s;
     };
     int32_t cap4 = 0, waves = 4;
-    int32_t s = plan(4, u8 && c.head_size > 128 ? 256 : 512, &cap4);
+    int32_t s = plan(4, c.head_size > 128 ? 256 : 512, &cap4);
     // A context whose probabilities do not fit half a CU's LDS is cut into splits that send every head's
     // probabilities through HBM and add a merge.  With enough (sequence, kv head) pairs to give every CU a workgroup
     // of its own, one workgroup of eight waves per CU (the same waves per CU, the whole LDS) needs fewer of them.
@@ -804,7 +806,7 @@ void do_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool static
         PA_REQUIRE((use_decode && (int32_t)ctx->h_dec.size() == ctx->B) || (use_decode16 && !mfma_left && !use_decode),
                    PA_NOT_IMPLEMENTED,
                    "pa_attention_static serves steps in which every sequence schedules one token, over a u8 cache or a "
-                   "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64 or 128, over u8 also 96 and -- from block size 32 -- 256, K and V alike; at most 16 heads per kv head)");
+                   "16-bit cache of the query's type (block size 16 to 256, a power of two; head size 64, 96, 128 or 256 -- over u8 with 16-token blocks not 256 --, K and V alike; at most 16 heads per kv head)");
     // the timed kernel: the matrix kernel when there is prefill work, else the decode kernel
     hipEvent_t ev0 = ctx->profiling ? ctx->ev0 : nullptr, ev1 = ctx->profiling ? ctx->ev1 : nullptr;
     // fork: what is launched on the returned stream starts behind what the context's stream holds so far and runs

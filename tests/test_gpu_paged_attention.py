@@ -324,6 +324,13 @@ DECODE16 = [
     ("bf16_d128_g5_odd_blocks", (10, 2, 128, 32, "bf16", "bf16", [4127, 95, 33], [1] * 3), {}),
     ("f16_d128_g5_long_splits", (5, 1, 128, 32, "f16", "f16", [12001], [1]), {}),
     ("f16_g17_stays_on_the_matrix_kernel", (17, 1, 64, 32, "f16", "f16", [200, 77], [1, 1]), {}),
+    # head sizes 96 and 256 (256: one workgroup per CU)
+    ("f16_d96_mha", (6, 6, 96, 32, "f16", "f16", [37, 130, 64, 4097, 0, 31, 32, 33], [1] * 8), {}),
+    ("bf16_d96_g3_bs16_long_splits", (12, 4, 96, 16, "bf16", "bf16", [9000, 4000], [1, 1]), {"sliding_window": 2500}),
+    ("bf16_d256_g2", (16, 8, 256, 32, "bf16", "bf16", [37, 130, 64, 4097, 0, 31, 32, 33], [1] * 8), {}),
+    ("f16_d256_g16_long_splits_bs64", (16, 1, 256, 64, "f16", "f16", [15000], [1]), {}),
+    ("f16_d256_bs16_window_inside_block", (4, 4, 256, 16, "f16", "f16", [100, 45, 700], [1] * 3), {"sliding_window": 40}),
+    ("f16_d96_g17_runs_on_the_generic_kernel", (17, 1, 96, 32, "f16", "f16", [200, 77], [1, 1]), {}),
 ]
 
 
@@ -490,6 +497,7 @@ LATE_APPEND = [
     ("f16", "f16", 32, 64, (1100, 1300)), ("bf16", "bf16", 16, 64, (1100, 1300)), ("bf16", "bf16", 32, 8, (20000, 33000)),
     # head size 256 (a seventh field: query heads, kv heads, head size)
     ("f16", "u8", 32, 64, (1100, 1300), (16, 8, 256)), ("bf16", "u8", 64, 8, (20000, 33000), (16, 8, 256)),
+    ("bf16", "bf16", 32, 64, (1100, 1300), (16, 8, 256)), ("f16", "f16", 16, 8, (20000, 33000), (12, 4, 96)),
 ]
 LATE_APPEND = [c if len(c) == 6 else c + ((32, 8, 128),) for c in LATE_APPEND]
 

@@ -1,6 +1,7 @@
 """Generators of random steps beyond the suite's own: longer contexts and chunks (``big``), logits scaled so that few
 tokens carry a row (``peaked``), decode steps that take the eight-wave plan of the u8 decode kernel (``wide``) and
-block-sparse prefill steps (``sparse``).  Used by ``test_gpu_soak_slice.py``."""
+block-sparse prefill steps (``sparse``), and steps at head sizes 96 and 256 (``heads``).  Used by
+``test_gpu_soak_slice.py``."""
 import numpy as np
 
 import harness as H
@@ -24,6 +25,29 @@ def big_case(rng, idx):
     bs = 16 if idx % 4 == 3 else 32  # (from the index, not the generator: the other cases stay what they were)
     return H.case_from_lens(f"big_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_sw{sw}_b{bs}", Hkv * G, Hkv, D, bs, qd, kd, past, new,
                             sliding_window=sw, score_aggregation_window=saw)
+
+
+def heads_case(rng, idx):
+    """Head sizes 96 and 256: the tuned kernels' instantiations with six value channels per lane / one workgroup per
+    CU (and, with more than 16 heads per kv head or 16-token blocks at 256 over u8, the shape-generic kernel)."""
+    D = int(rng.choice([96, 256])); Hkv = int(rng.choice([1, 2, 8])); G = int(rng.choice([1, 2, 3, 4, 8, 16, 20]))
+    qd = str(rng.choice(["f16", "bf16"])); kd = str(rng.choice(["u8", "u8", qd]))
+    bs = int(rng.choice([16, 32, 32, 32, 64, 128]))
+    B = int(rng.integers(1, 9))
+    kind = rng.choice(["decode", "decode", "prefill", "mixed"])
+    past, new = [], []
+    for _ in range(B):
+        if kind == "decode" or (kind == "mixed" and rng.random() < 0.6):
+            past.append(int(rng.choice([int(rng.integers(0, 2000)), int(rng.integers(2000, 9000))])))
+            new.append(1)
+        else:
+            past.append(int(rng.choice([0, int(rng.integers(1, 4000))])))
+            new.append(int(rng.integers(2, 400)))
+    sw = int(rng.choice([0, 0, 0, int(rng.integers(40, 3000))]))
+    saw = [int(rng.integers(0, min(n, 16) + 1)) for n in new] if rng.random() < 0.7 else None
+    mult = float(rng.choice([1.0, 1.0, 1.0, 4.0]))
+    return H.case_from_lens(f"heads_{idx}_{kind}_{qd}_{kd}_D{D}_H{Hkv}x{G}_sw{sw}_b{bs}_x{mult}", Hkv * G, Hkv, D, bs, qd, kd,
+                            past, new, sliding_window=sw, score_aggregation_window=saw, scale=mult / np.sqrt(D))
 
 
 def peaked_case(rng, idx):

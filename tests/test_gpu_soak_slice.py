@@ -10,7 +10,8 @@ import test_gpu_xattention as TX
 
 pytestmark = pytest.mark.gpu
 
-KINDS = {"small": T._random_case, "big": S.big_case, "peaked": S.peaked_case, "wide": S.wide_case, "sparse": S.sparse_case}
+KINDS = {"small": T._random_case, "big": S.big_case, "peaked": S.peaked_case, "wide": S.wide_case, "sparse": S.sparse_case,
+         "heads": S.heads_case}
 
 
 @pytest.fixture(scope="module")

@@ -151,8 +151,7 @@ typedef struct pa_layer_io {
  * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
  * writes).  Head sizes 96 and 256 (K and V alike, the same caches) run on instantiations of the same kernels with
  * these limits: the matrix kernel keeps to 16 query rows per wave, block-sparse prefill is not offered, the u8 decode
- * kernel does not take head size 256 with 16-token blocks (such steps run on the shape-generic kernel), and at head
- * size 96 the append of a step's rows over a u8 cache is always a launch of its own. */
+ * kernel does not take head size 256 with 16-token blocks (such steps run on the shape-generic kernel). */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The op's `alibi_slopes` input (input 11: f32 [num_heads]; a graph constant that SDPAToPagedAttention leaves empty
  * for models without ALiBi, and that the reference never sets itself): with slopes set, every logit gets

@@ -123,7 +123,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 2) void pa_decode_u8_kern
     constexpr int NW = (VB + 3) / 4;       // ... held in this many 32-bit words
     constexpr int SLOT = TILE;             // a wave's LDS staging slot: a K block, then a V block
     constexpr int EPL = (D + 63) / 64;     // elements per lane of a new K / V row
-    constexpr bool CAN_APPEND = D % 64 == 0;  // (a row of the fused append is spread over all 64 lanes)
+    constexpr int ROW_LANES = D / EPL;     // lanes a new row spreads over (D = 96: 48, the others repeat lanes 32 - 47)
     constexpr int DEPTH = 2;               // blocks a wave keeps in flight
     // Channel of row m of output tile r (the lane with n = m reads that channel's byte of each of its token rows): a
     // lane's VB consecutive channels, except that with 6 bytes per lane (D = 96) the lanes take four consecutive
@@ -161,18 +161,17 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 2) void pa_decode_u8_kern
     // see the row, and loads and stores of a wave may complete out of order with respect to each other, so the wave
     // waits for its stores explicitly (vmcnt(0)) before it issues the fetch of that block: at once when the block is
     // among its first ones, else (the stores then follow its first fetches) right in front of that fetch.
-    const bool appends = CAN_APPEND && a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
+    const bool appends = a.fuse_append && te == tile_hi && te > tb && (tile_hi - 1 - tb) % WAVES == wv;
     const bool append_first = appends && tile_hi - 1 - tb < 4 * WAVES;
     auto append_rows = [&]() __attribute__((always_inline)) {
-        if constexpr (CAN_APPEND) {
-            const long src = ((long)t * Hkv + hkv) * D + lane * EPL;
-            const long dst = (((long)dsc->last_id * Hkv + hkv) * bsz + (kv_len - 1) % bsz) * ROW;
-            uint16_t kr[EPL], vr[EPL];
-            load_row16<EPL>(a.key + src, kr);
-            load_row16<EPL>(a.value + src, vr);
-            quantize_row_u8<QDT, EPL>(kr, const_cast<uint8_t*>(a.key_cache) + dst, lane);
-            quantize_row_u8<QDT, EPL>(vr, const_cast<uint8_t*>(a.value_cache) + dst, lane);
-        }
+        const int rl = lane < ROW_LANES ? lane : lane - (64 - ROW_LANES);
+        const long src = ((long)t * Hkv + hkv) * D + rl * EPL;
+        const long dst = (((long)dsc->last_id * Hkv + hkv) * bsz + (kv_len - 1) % bsz) * ROW;
+        uint16_t kr[EPL], vr[EPL];
+        load_row16<EPL>(a.key + src, kr);
+        load_row16<EPL>(a.value + src, vr);
+        quantize_row_u8<QDT, EPL>(kr, const_cast<uint8_t*>(a.key_cache) + dst, rl, lane < ROW_LANES);
+        quantize_row_u8<QDT, EPL>(vr, const_cast<uint8_t*>(a.value_cache) + dst, rl, lane < ROW_LANES);
     };
     if (append_first) {
         append_rows();

@@ -98,9 +98,11 @@ __device__ __forceinline__ float row16_sum(float v) {
 //   scale = (max - min) / 255  (a zero range takes 1e-4),  zp = -min / scale,
 //   code  = clamp(rne(fma(x, 1/scale, zp)), 0, 255),
 // every operation in IEEE binary32 (no contraction), so that the bytes are reproducible on any IEEE host.
-// `raw` holds the lane's EPL consecutive elements (bit patterns of QDT); `dst` is the row's first byte.
+// `raw` holds the lane's EPL consecutive elements (bit patterns of QDT), elements lane * EPL ..; `dst` is the row's
+// first byte.  A row shorter than 64 * EPL elements: the surplus lanes hold copies of other lanes' elements (which
+// leaves minimum and maximum alone), pass those lanes' numbers and `store` = false.
 template <int QDT, int EPL>
-__device__ __forceinline__ void quantize_row_u8(const uint16_t (&raw)[EPL], uint8_t* dst, const int lane) {
+__device__ __forceinline__ void quantize_row_u8(const uint16_t (&raw)[EPL], uint8_t* dst, const int lane, const bool store = true) {
 #pragma clang fp contract(off)
     float x[EPL];
 #pragma unroll
@@ -121,6 +123,7 @@ __device__ __forceinline__ void quantize_row_u8(const uint16_t (&raw)[EPL], uint
         v = fminf(fmaxf(v, 0.0f), 255.0f);
         packed |= (uint32_t)(int)v << (8 * e);
     }
+    if (!store) return;
     if (lane == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
     uint8_t* c = dst + 8 + lane * EPL;
     if constexpr (EPL == 4) *reinterpret_cast<uint32_t*>(c) = packed;

@@ -352,8 +352,6 @@ bool decode_u8_shape(const pa_config& c) {
            (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || (c.head_size == 256 && c.block_size >= 32)) &&
            c.num_heads / c.num_kv_heads <= 16;
 }
-// ... and whose rows the decode kernels can append themselves (a row spread over all 64 lanes).
-bool fused_append_shape(const pa_config& c) { return c.head_size % 64 == 0; }
 
 // Shapes the MFMA kernel is built for: 16-bit caches of the query's type, or u8 caches (dequantised on the way to
 // LDS).  It takes every sequence the decode kernel does not.
@@ -1489,7 +1487,7 @@ int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io) {
         HIP_CHECK(hipSetDevice(ctx->cfg.device));
         // a step of single-token sequences that all go to one of the decode kernels: it appends the new rows itself
         const bool fuse = ctx->step_ready &&
-                          ((decode_u8_shape(ctx) && fused_append_shape(ctx->cfg) && (int32_t)ctx->h_dec.size() == ctx->B) ||
+                          ((decode_u8_shape(ctx) && (int32_t)ctx->h_dec.size() == ctx->B) ||
                            (mfma_shape(ctx) && decode16_shape(ctx) && (int32_t)ctx->h_dec16.size() == ctx->B &&
                             ctx->n_sparse == 0 && ctx->n_single == ctx->n_items));
         if (fuse) check_io(ctx, layer, io, true, false);

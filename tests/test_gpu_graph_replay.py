@@ -12,6 +12,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("kv,past,new", [("u8", [700, 64, 1300, 31], [1, 1, 1, 1]),       # decode kernel, one split
                                          ("u8", [9000], [1]),                             # several splits + merge
                                          ("bf16", [300, 40, 0], [1, 1, 70]),              # matrix kernel, mixed step
+                                         ("u8", [300, 40, 0], [1, 1, 70]),                # decode kernel on the second stream beside the matrix kernel
                                          ("bf16", [700, 64, 1300, 31], [1, 1, 1, 1]),     # 16-bit decode kernel (appends too)
                                          ("bf16", [9000, 20], [1, 1])])                   # the same with several splits
 def test_graph_replays_equal_eager(pkg, kv, past, new):

@@ -498,6 +498,7 @@ LATE_APPEND = [
     # head size 256 (a seventh field: query heads, kv heads, head size)
     ("f16", "u8", 32, 64, (1100, 1300), (16, 8, 256)), ("bf16", "u8", 64, 8, (20000, 33000), (16, 8, 256)),
     ("bf16", "bf16", 32, 64, (1100, 1300), (16, 8, 256)), ("f16", "f16", 16, 8, (20000, 33000), (12, 4, 96)),
+    ("f16", "u8", 32, 64, (1100, 1300), (12, 4, 96)), ("bf16", "u8", 16, 8, (20000, 33000), (6, 6, 96)),
 ]
 LATE_APPEND = [c if len(c) == 6 else c + ((32, 8, 128),) for c in LATE_APPEND]
 

@@ -563,8 +563,10 @@ void plan_items(pa_ctx* ctx) {
     ctx->h_dec.clear();
     ctx->h_dec16.clear();
     // A mixed step over a 16-bit cache with the 16-bit decode kernel available: chunk items and single-token
-    // sequences do not share a launch -- the chunks go to the straight-to-LDS variant, the single-token sequences to
-    // the decode kernel on a second stream, side by side.  Their items are still listed (behind the chunks' items, where
+    // sequences do not share a launch -- the chunks go to the straight-to-LDS variant (head size 128; else the
+    // one-row-group variant), the single-token sequences to the decode kernel on a second stream, side by side
+    // (60 single tokens at 512 - 8192 positions beside four 512-token chunks over f16, against one launch for both:
+    // head size 128 0.296 -> 0.283 ms, 64 0.226 -> 0.213, 96 0.806 -> 0.787; at 256 no difference, left as one launch).  Their items are still listed (behind the chunks' items, where
     // the matrix kernel passes them over) but count for nothing in the plan of the chunks.
     {
         bool any_single = false, any_chunk = false;
@@ -573,7 +575,7 @@ void plan_items(pa_ctx* ctx) {
             any_single = any_single || q_len == 1;
             any_chunk = any_chunk || (q_len > 1 && xatt_seq_index(ctx, b) < 0);
         }
-        ctx->split16 = narrow_all && any_single && any_chunk && decode16_shape(ctx) && ctx->cfg.head_size == 128;
+        ctx->split16 = narrow_all && any_single && any_chunk && decode16_shape(ctx) && ctx->cfg.head_size != 256;
     }
     size_t planned_tiles = 0;
     for (int32_t b = 0; b < B; ++b) {

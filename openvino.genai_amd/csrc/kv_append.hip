@@ -33,9 +33,9 @@ __device__ __forceinline__ void append_row(uint32_t (&w)[E / 2], uint8_t* dst, i
         if (scale == 0.0f) scale = 0.0001f;
         const float zp = -mn / scale;
         const float inv = 1.0f / scale;
-        uint32_t codes[E / 4];
+        uint32_t codes[(E + 3) / 4];
 #pragma unroll
-        for (int i = 0; i < E / 4; ++i) codes[i] = 0;
+        for (int i = 0; i < (E + 3) / 4; ++i) codes[i] = 0;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             float v = rintf(__fmaf_rn(x[e], inv, zp));
@@ -45,7 +45,11 @@ __device__ __forceinline__ void append_row(uint32_t (&w)[E / 2], uint8_t* dst, i
         if (l16 == 0) *reinterpret_cast<float2*>(dst) = make_float2(scale, zp);
         uint8_t* c = dst + 8 + l16 * E;  // rows are multiples of 8 bytes
         if constexpr (E == 4) *reinterpret_cast<uint32_t*>(c) = codes[0];
-        else
+        else if constexpr (E == 6) {  // (a lane's six bytes start on a 2-byte boundary)
+            reinterpret_cast<uint16_t*>(c)[0] = (uint16_t)codes[0];
+            reinterpret_cast<uint16_t*>(c)[1] = (uint16_t)(codes[0] >> 16);
+            reinterpret_cast<uint16_t*>(c)[2] = (uint16_t)codes[1];
+        } else
 #pragma unroll
             for (int i = 0; i < E / 8; ++i) *reinterpret_cast<uint2*>(c + 8 * i) = make_uint2(codes[2 * i], codes[2 * i + 1]);
     } else {
@@ -57,7 +61,10 @@ __device__ __forceinline__ void append_row(uint32_t (&w)[E / 2], uint8_t* dst, i
         }
         uint8_t* c = dst + l16 * E * 2;
         if constexpr (E == 4) *reinterpret_cast<uint2*>(c) = make_uint2(w[0], w[1]);
-        else
+        else if constexpr (E == 6) {  // (twelve bytes on a 4-byte boundary)
+#pragma unroll
+            for (int i = 0; i < 3; ++i) reinterpret_cast<uint32_t*>(c)[i] = w[i];
+        } else
 #pragma unroll
             for (int i = 0; i < E / 8; ++i) *reinterpret_cast<uint4*>(c + 16 * i) = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
     }
@@ -68,6 +75,9 @@ __device__ __forceinline__ void load_row(uint32_t (&w)[E / 2], const uint16_t* s
     if constexpr (E == 4) {
         const uint2 v = *reinterpret_cast<const uint2*>(src);
         w[0] = v.x; w[1] = v.y;
+    } else if constexpr (E == 6) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) w[i] = reinterpret_cast<const uint32_t*>(src)[i];
     } else {
 #pragma unroll
         for (int i = 0; i < E / 8; ++i) {
@@ -77,7 +87,8 @@ __device__ __forceinline__ void load_row(uint32_t (&w)[E / 2], const uint16_t* s
     }
 }
 
-// A row per 16 lanes, each lane D / 16 consecutive elements (16-byte loads at D = 128), four rows per wave.  A wave
+// A row per 16 lanes, each lane D / 16 consecutive elements (16-byte loads at D = 128 and 256, 4-byte ones at 96),
+// four rows per wave.  A wave
 // takes four consecutive tokens of one kv head, so that what it writes is one run of cache bytes wherever the
 // tokens share a block.  Minimum and maximum of a row are reduced over its 16 lanes with four
 // cross-lane (DPP) steps; the arithmetic per element is that of quantize_row_u8, so the bytes are the same.
@@ -88,7 +99,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(StepDev st, Shape sh, co
                                                         uint8_t* __restrict__ value_cache,
                                                         const int32_t* __restrict__ block_indices) {
 #pragma clang fp contract(off)
-    static_assert(E == 4 || E == 8, "D = 64 or 128");
+    static_assert(E == 4 || E == 6 || E == 8 || E == 16, "D = 64, 96, 128 or 256");
     constexpr int D = 16 * E;
     const int l16 = threadIdx.x & 15;
     const long per_tensor = (long)st.T * sh.Hkv;
@@ -121,7 +132,7 @@ __global__ __launch_bounds__(256) void kv_append_tokens_kernel(StepDev st, Shape
                                                                uint8_t* __restrict__ key_cache,
                                                                uint8_t* __restrict__ value_cache,
                                                                const int32_t* __restrict__ block_indices) {
-    static_assert(E == 4 || E == 8, "D = 64 or 128");
+    static_assert(E == 4 || E == 6 || E == 8 || E == 16, "D = 64, 96, 128 or 256");
     constexpr int D = 16 * E, U = 4;
     constexpr int RB = KVDT == DT_U8 ? D + 8 : 2 * D;
     const int l16 = threadIdx.x & 15;
@@ -164,16 +175,20 @@ hipError_t launch_epl(hipStream_t s, const StepDev& st, const Shape& sh, const v
     auto vcu = reinterpret_cast<uint8_t*>(vc);
     if (st.T >= TOKENS_KERNEL_MIN_T) {  // enough tokens to fill the chip with a token per 16 lanes
         const dim3 tgrid((unsigned)((st.T + 15) / 16));
-        switch (sh.D / 64) {
-            case 1: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 4>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
-            case 2: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 8>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        switch (sh.D) {
+            case 64: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 4>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+            case 96: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 6>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+            case 128: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 8>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+            case 256: hipLaunchKernelGGL((kv_append_tokens_kernel<QDT, KVDT, 16>), tgrid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
             default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
     }
-    switch (sh.D / 64) {
-        case 1: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 4>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
-        case 2: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 8>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+    switch (sh.D) {
+        case 64: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 4>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        case 96: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 6>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        case 128: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 8>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
+        case 256: hipLaunchKernelGGL((kv_append_kernel<QDT, KVDT, 16>), grid, block, 0, s, st, sh, k, v, kcu, vcu, bi); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -267,9 +267,11 @@ pa::Shape shape_of(const pa_config& c) { return pa::Shape{c.num_heads, c.num_kv_
 pa::GenericShape generic_shape_of(const pa_config& c) {
     return pa::GenericShape{c.num_heads, c.num_kv_heads, c.head_size, v_head(c), c.block_size, c.kv_cache_dtype, v_dtype(c)};
 }
-// The append kernel with a row per 16 lanes is built for K and V alike, head size 64 or 128; everything else takes the
+// The append kernel with a row per 16 lanes is built for K and V alike, head size 64, 96, 128 or 256; everything else takes the
 // shape-generic one (a wave per row).
-bool tuned_append_shape(const pa_config& c) { return kv_alike(c) && (c.head_size == 64 || c.head_size == 128); }
+bool tuned_append_shape(const pa_config& c) {
+    return kv_alike(c) && (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || c.head_size == 256);
+}
 
 const int32_t* table_for(pa_ctx* ctx, int32_t layer) {
     PA_REQUIRE(layer >= 0 && layer < ctx->cfg.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");

@@ -22,11 +22,17 @@ CONFIGS = {
     # long-context decode, 32B-class shape, batch 8 x 32768 (variant: sliding window 4096)
     5: dict(name="long_context_decode_u8_b8_ctx32768", Hq=40, Hkv=8, D=128, bs=32, q_dtype="f16", kv_dtype="u8", B=8,
             past=("const", 32768), new=1, sliding_window=0),
+    # diagnostics beyond the five benchmark workloads: the headline step at the other head sizes the tuned kernels
+    # are instantiated for (Phi-3-mini-like: 32 heads without grouping, head size 96; Gemma-2-9B-like: 16 / 8, 256)
+    6: dict(name="phi3_mini_decode_u8_b64_ctx4096", Hq=32, Hkv=32, D=96, bs=32, q_dtype="f16", kv_dtype="u8", B=64,
+            past=("const", 4096), new=1, sliding_window=0),
+    7: dict(name="gemma2_9b_decode_u8_b64_ctx4096", Hq=16, Hkv=8, D=256, bs=32, q_dtype="f16", kv_dtype="u8", B=64,
+            past=("const", 4096), new=1, sliding_window=0),
 }
 
 
 def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0, block_size=None):
-    """Step metadata of config ``cfg`` (1..5); ``batch`` / ``context_scale`` shrink it for parity tests."""
+    """Step metadata of config ``cfg`` (1..7); ``batch`` / ``context_scale`` shrink it for parity tests."""
     c = dict(CONFIGS[cfg])
     rng = np.random.Generator(np.random.PCG64(1000 + cfg if seed is None else seed))
     B = c["B"] if batch is None else batch

@@ -60,7 +60,9 @@ def _check_whole_batch(spec, q, kc, vc, out, scores, W, qd, kd, sw):
 
 
 APPEND_CASES = [("f16", "u8", 128), ("f16", "u8", 64), ("bf16", "u8", 128), ("f16", "f16", 64), ("bf16", "bf16", 128),
-                ("f16", "bf16", 128), ("bf16", "f16", 64)]
+                ("f16", "bf16", 128), ("bf16", "f16", 64),
+                ("f16", "u8", 96), ("bf16", "u8", 256), ("f16", "f16", 96), ("bf16", "bf16", 256), ("f16", "bf16", 96),
+                ("bf16", "f16", 256)]
 
 
 @pytest.mark.parametrize("qd,kd,D", APPEND_CASES)
@@ -74,7 +76,8 @@ MANY_ROWS = [
     # append kernel with a row per 16 lanes
     ("f16", "u8", 128, 4, 32), ("bf16", "u8", 128, 8, 32), ("f16", "u8", 64, 4, 32), ("bf16", "u8", 64, 2, 32),
     ("f16", "u8", 128, 4, 16), ("f16", "f16", 128, 4, 32), ("bf16", "bf16", 64, 4, 32), ("f16", "bf16", 128, 4, 32),
-    ("bf16", "f16", 64, 2, 16),
+    ("bf16", "f16", 64, 2, 16), ("f16", "u8", 96, 4, 32), ("bf16", "u8", 256, 2, 32), ("f16", "f16", 96, 3, 16),
+    ("bf16", "bf16", 256, 2, 64),
 ]
 
 
@@ -89,6 +92,7 @@ MANY_TOKENS = [
     # time (3 kv heads: the last group of rows is not full)
     ("f16", "u8", 128, 8, 32), ("bf16", "u8", 64, 3, 32), ("f16", "u8", 128, 1, 16), ("bf16", "bf16", 128, 4, 32),
     ("f16", "bf16", 64, 3, 64), ("bf16", "f16", 128, 2, 32),
+    ("f16", "u8", 96, 3, 32), ("bf16", "u8", 256, 2, 32), ("bf16", "bf16", 96, 2, 16), ("f16", "f16", 256, 1, 64),
 ]
 
 

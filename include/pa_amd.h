@@ -65,7 +65,7 @@ typedef struct pa_config {
     int32_t device;          /* HIP device ordinal */
     int32_t num_heads;       /* query heads */
     int32_t num_kv_heads;    /* KV heads; num_heads must be a multiple */
-    int32_t head_size;       /* elements of a query / key row: a multiple of 8 up to 512 (64 and 128 have tuned kernels) */
+    int32_t head_size;       /* elements of a query / key row: a multiple of 8 up to 512 (64, 96, 128 and 256 have tuned kernels) */
     int32_t block_size;      /* tokens per KV block: the reference fixes 32 on CPU, 16 on GPU
                                 (kv_cache_manager.hpp:97-110); here a knob */
     int32_t query_dtype;     /* PA_F16 | PA_BF16: query, key, value and the output */

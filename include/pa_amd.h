@@ -174,7 +174,9 @@ int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
  * PA_NOT_IMPLEMENTED.  The split partials,
  * final maxima / denominators and the score staging live in a fixed device array of PA_STATIC_SCRATCH_BYTES bytes
  * (32 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls
- * no hipMalloc / hipFree; a step that needs more returns PA_OUT_OF_BOUNDS and a message with the byte count.  (The
+ * no hipMalloc / hipFree, and the device code of its kernels is uploaded by pa_create, not by the first call (the
+ * runtime would otherwise allocate for it inside that call); a step that needs more returns PA_OUT_OF_BOUNDS and a
+ * message with the byte count.  (The
  * step arrays and block tables are uploaded -- and their buffers grown -- by pa_step_begin / pa_set_block_indices,
  * as for pa_attention.)  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race, also from
  * different contexts; calls in stream order on one stream do not.  Nothing in it needs clearing between calls: each

@@ -427,6 +427,11 @@ size_t decode16_lds_bytes(int D, int G, int max_tiles, bool want_scores) {
     return (bytes + 15) & ~(size_t)15;
 }
 
+hipError_t preload_decode16() {  // (see preload_decode_u8)
+    hipFuncAttributes at;
+    return hipFuncGetAttributes(&at, reinterpret_cast<const void*>(pa_decode16_kernel<128, DT_F16, 32>));
+}
+
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,
                            hipEvent_t ev1) {
     if (a.sh.bs < 16 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1)) || a.G > 16 || (a.want_scores != 0) != (scores != nullptr)) return hipErrorInvalidValue;

@@ -797,6 +797,13 @@ hipError_t launch_decode_post(hipStream_t s, const DecodeArgs& a, int q_dtype, f
     return scores ? launch_decode_scores(s, a, scores, max_kv_len) : hipSuccess;
 }
 
+// The runtime uploads a translation unit's device code when one of its kernels is first asked for; asking here, when
+// a context is created, keeps that allocation out of the first attention call.
+hipError_t preload_decode_u8() {
+    hipFuncAttributes at;
+    return hipFuncGetAttributes(&at, reinterpret_cast<const void*>(pa_decode_u8_kernel<128, DT_F16, 4, 32>));
+}
+
 hipError_t launch_decode_u8(hipStream_t s, const DecodeArgs& a, int q_dtype, float* scores, int max_kv_len,
                             hipEvent_t ev0, hipEvent_t ev1) {
     if (a.sh.D == 128)

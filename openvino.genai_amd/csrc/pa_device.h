@@ -305,6 +305,8 @@ size_t decode16_table_bytes(int max_tiles, int block_size);  // the block-table 
 hipError_t launch_decode16(hipStream_t s, const DecodeArgs& a, int dtype, float* scores, int max_kv_len, hipEvent_t ev0,
                            hipEvent_t ev1);
 // The merge and score kernels of the decode family on their own.
+hipError_t preload_decode_u8();
+hipError_t preload_decode16();
 hipError_t launch_decode_merge(hipStream_t s, const DecodeArgs& a, int q_dtype);
 hipError_t launch_decode_scores(hipStream_t s, const DecodeArgs& a, float* scores, int max_kv_len);
 hipError_t launch_decode_post(hipStream_t s, const DecodeArgs& a, int q_dtype, float* scores, int max_kv_len);

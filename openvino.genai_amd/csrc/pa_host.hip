@@ -1022,6 +1022,10 @@ int32_t pa_create(const pa_config* cfg, pa_ctx** out) {
         check_config(cfg);
         HIP_CHECK(hipSetDevice(cfg->device));
         uint8_t* fixed = static_cast<uint8_t*>(resolve_static_scratch(cfg->device));
+        // the decode kernels' device code is uploaded now rather than inside the first attention call (which, for
+        // pa_attention_static, must not allocate)
+        HIP_CHECK(pa::preload_decode_u8());
+        HIP_CHECK(pa::preload_decode16());
         pa_ctx* ctx = new pa_ctx();
         ctx->cfg = *cfg;
         ctx->stream = static_cast<hipStream_t>(cfg->stream);

@@ -33,17 +33,19 @@ def _run(torch, op, case, dev, static, want_scores=True):
             op.num_splits)
 
 
-@pytest.mark.parametrize("kv_dtype,q_dtype", [("u8", "f16"), ("bf16", "bf16")])
-def test_static_entry_point_matches_pa_attention_on_two_calls_in_a_row(pkg, kv_dtype, q_dtype):
+@pytest.mark.parametrize("kv_dtype,q_dtype,heads", [("u8", "f16", (32, 8, 128)), ("bf16", "bf16", (32, 8, 128)),
+                                                    ("u8", "bf16", (16, 8, 256)), ("f16", "f16", (12, 4, 96))])
+def test_static_entry_point_matches_pa_attention_on_two_calls_in_a_row(pkg, kv_dtype, q_dtype, heads):
     """Two calls in a row on the shared scratch, the second with a smaller input: outputs and scores are those of
     pa_attention bit for bit (same kernels, other workspace) and within tolerance of the CPU checker."""
     import torch
     dev = torch.device("cuda:0")
-    big = H.build_case(H.case_from_lens("static_big", 32, 8, 128, 32, q_dtype, kv_dtype,
+    Hq, Hkv, D = heads
+    big = H.build_case(H.case_from_lens("static_big", Hq, Hkv, D, 32, q_dtype, kv_dtype,
                                         [9000, 4500, 7000, 123, 8100, 6400], [1] * 6), seed=11)
-    small = H.build_case(H.case_from_lens("static_small", 32, 8, 128, 32, q_dtype, kv_dtype, [700, 33, 1500], [1] * 3), seed=12)
-    ref_op = pkg.PagedAttention(32, 8, 128, 32, q_dtype, kv_dtype, 1, 0, torch.cuda.current_stream(dev))
-    st_op = pkg.PagedAttention(32, 8, 128, 32, q_dtype, kv_dtype, 1, 0, torch.cuda.current_stream(dev))
+    small = H.build_case(H.case_from_lens("static_small", Hq, Hkv, D, 32, q_dtype, kv_dtype, [700, 33, 1500], [1] * 3), seed=12)
+    ref_op = pkg.PagedAttention(Hq, Hkv, D, 32, q_dtype, kv_dtype, 1, 0, torch.cuda.current_stream(dev))
+    st_op = pkg.PagedAttention(Hq, Hkv, D, 32, q_dtype, kv_dtype, 1, 0, torch.cuda.current_stream(dev))
     splits = []
     for case in (big, small):  # the static calls follow each other on the same scratch
         out_s, sc_s, ns = _run(torch, st_op, case, dev, static=True)
@@ -57,7 +59,7 @@ def test_static_entry_point_matches_pa_attention_on_two_calls_in_a_row(pkg, kv_d
         qd, kd = H.DT[q_dtype], H.DT[kv_dtype]
         out, out16, scores = O.paged_attention(case["query"], qd, case["key_cache0"], case["value_cache0"], kd,
                                                case["past_lens"], case["subsequence_begins"], case["block_indices"],
-                                               case["block_indices_begins"], 32, 8, 128, 32, case["scale"], 0, None, True, 8)
+                                               case["block_indices_begins"], Hq, Hkv, D, 32, case["scale"], 0, None, True, 8)
         H.assert_close(O.from_bits(out_s, qd), out, q_dtype)
         H.assert_close(sc_s, scores, "f16", "scores")
     assert splits[0] > 1, "the first case is meant to use the split partials of the scratch"

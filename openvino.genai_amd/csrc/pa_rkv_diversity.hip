@@ -52,15 +52,24 @@ __device__ __forceinline__ f4 mma(const s8v& a, const s8v& b, const f4& c) {
 template <int D, int KVDT>
 __device__ __forceinline__ void lane_channels(const uint8_t* row, int l16, float (&x)[D / 16], float (&code)[D / 16]) {
     constexpr int E = D / 16;
+    static_assert(E == 4 || E == 6 || E == 8 || E == 16, "head size 64, 96, 128 or 256");
     if (KVDT == DT_U8) {
         const float2 hd = *reinterpret_cast<const float2*>(row);
-        uint32_t w[E / 4];
-        if constexpr (E == 8) {
-            const u2v v = *reinterpret_cast<const u2v*>(row + 8 + 8 * l16);
+        uint32_t w[(E + 3) / 4];
+        const uint8_t* p = row + 8 + E * l16;
+        if constexpr (E == 16) {  // (rows start on 8-byte boundaries)
+            const u2v v0 = *reinterpret_cast<const u2v*>(p), v1 = *reinterpret_cast<const u2v*>(p + 8);
+            w[0] = v0[0], w[1] = v0[1], w[2] = v1[0], w[3] = v1[1];
+        } else if constexpr (E == 8) {
+            const u2v v = *reinterpret_cast<const u2v*>(p);
             w[0] = v[0];
             w[1] = v[1];
+        } else if constexpr (E == 6) {  // (six bytes on a 2-byte boundary)
+            const uint16_t* h = reinterpret_cast<const uint16_t*>(p);
+            w[0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+            w[1] = h[2];
         } else {
-            w[0] = *reinterpret_cast<const uint32_t*>(row + 8 + 4 * l16);
+            w[0] = *reinterpret_cast<const uint32_t*>(p);
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
@@ -69,12 +78,19 @@ __device__ __forceinline__ void lane_channels(const uint8_t* row, int l16, float
         }
     } else {
         uint32_t w[E / 2];
-        if constexpr (E == 8) {
-            const u4v v = *reinterpret_cast<const u4v*>(row + 16 * l16);
+        const uint8_t* p = row + 2 * E * l16;
+        if constexpr (E % 8 == 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) w[i] = v[i];
+            for (int j = 0; j < E / 8; ++j) {
+                const u4v v = *reinterpret_cast<const u4v*>(p + 16 * j);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w[4 * j + i] = v[i];
+            }
+        } else if constexpr (E == 6) {  // (twelve bytes on a 4-byte boundary)
+#pragma unroll
+            for (int i = 0; i < 3; ++i) w[i] = reinterpret_cast<const uint32_t*>(p)[i];
         } else {
-            const u2v v = *reinterpret_cast<const u2v*>(row + 8 * l16);
+            const u2v v = *reinterpret_cast<const u2v*>(p);
             w[0] = v[0];
             w[1] = v[1];
         }
@@ -416,10 +432,15 @@ hipError_t launch_typed(hipStream_t s, const RkvDivArgs& a, int nseq, int ev_max
                        block, 0, s, a);
     // four row blocks per wave once that still leaves a few thousand waves
     const long waves4 = (long)nseq * ceil_div(ev_max, 128) * ceil_div(ev_max, 64);
-    if (waves4 >= 4096)
-        hipLaunchKernelGGL((rkv_diversity_kernel<D, DT, KVDT == DT_U8, 4>),
-                           dim3((unsigned)ceil_div(ev_max, 256), (unsigned)ceil_div(ev_max, 128), (unsigned)nseq), block, 0, s, a);
-    else
+    // (head size 256: the columns' operands alone are 128 registers, four row blocks would spill)
+    bool four = false;
+    if constexpr (D <= 128) {
+        four = waves4 >= 4096;
+        if (four)
+            hipLaunchKernelGGL((rkv_diversity_kernel<D, DT, KVDT == DT_U8, 4>),
+                               dim3((unsigned)ceil_div(ev_max, 256), (unsigned)ceil_div(ev_max, 128), (unsigned)nseq), block, 0, s, a);
+    }
+    if (!four)
         hipLaunchKernelGGL((rkv_diversity_kernel<D, DT, KVDT == DT_U8, 1>),
                            dim3((unsigned)ceil_div(ev_max, 256), (unsigned)(ev_max / 32), (unsigned)nseq), block, 0, s, a);
     return hipGetLastError();
@@ -432,15 +453,17 @@ int rkv_diversity_chunks(int ev_max) { return ceil_div(ev_max, CHUNK); }
 hipError_t launch_rkv_diversity(hipStream_t s, const RkvDivArgs& a, int kv_dtype, int D, int bs, int nseq, int ev_max) {
     if (nseq == 0 || ev_max == 0) return hipSuccess;
     if (bs != 32 || ev_max % 32) return hipErrorInvalidValue;
-    if (D == 128) {
-        if (kv_dtype == DT_U8) return launch_typed<128, DT_U8>(s, a, nseq, ev_max);
-        if (kv_dtype == DT_F16) return launch_typed<128, DT_F16>(s, a, nseq, ev_max);
-        if (kv_dtype == DT_BF16) return launch_typed<128, DT_BF16>(s, a, nseq, ev_max);
-    } else if (D == 64) {
-        if (kv_dtype == DT_U8) return launch_typed<64, DT_U8>(s, a, nseq, ev_max);
-        if (kv_dtype == DT_F16) return launch_typed<64, DT_F16>(s, a, nseq, ev_max);
-        if (kv_dtype == DT_BF16) return launch_typed<64, DT_BF16>(s, a, nseq, ev_max);
+#define PA_DIV(D_)                                                                        \
+    if (D == D_) {                                                                        \
+        if (kv_dtype == DT_U8) return launch_typed<D_, DT_U8>(s, a, nseq, ev_max);        \
+        if (kv_dtype == DT_F16) return launch_typed<D_, DT_F16>(s, a, nseq, ev_max);      \
+        if (kv_dtype == DT_BF16) return launch_typed<D_, DT_BF16>(s, a, nseq, ev_max);    \
     }
+    PA_DIV(128)
+    PA_DIV(64)
+    PA_DIV(96)
+    PA_DIV(256)
+#undef PA_DIV
     return hipErrorInvalidValue;
 }
 

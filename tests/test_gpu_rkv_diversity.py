@@ -52,7 +52,7 @@ def _run(pkg, kv, q, Hq, Hkv, D, lens, start, ev_sizes, seed, keys=None):
 
 
 @pytest.mark.parametrize("kv,q", [("u8", "f16"), ("f16", "f16"), ("bf16", "bf16"), ("u8", "bf16")])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 96, 256])
 def test_diversity_matches_checker(pkg, kv, q, D):
     # areas: a multiple of 256 columns, tails of 32 / 96 columns, a sequence without a request, a single block
     lens = [700, 420, 333, 97, 1100]
@@ -62,7 +62,8 @@ def test_diversity_matches_checker(pkg, kv, q, D):
     assert max(np.abs(r).max() for _, r in res) > 1.0
 
 
-@pytest.mark.parametrize("kv,q,D", [("u8", "f16", 128), ("bf16", "bf16", 64), ("f16", "f16", 128)])
+@pytest.mark.parametrize("kv,q,D", [("u8", "f16", 128), ("bf16", "bf16", 64), ("f16", "f16", 128), ("u8", "bf16", 96),
+                                    ("f16", "f16", 256), ("u8", "f16", 256)])
 def test_diversity_of_long_areas(pkg, kv, q, D):
     """Areas long enough for the launch that gives a workgroup four row blocks (the one the benchmark measures): a
     whole number of 128-row groups, an area whose last group holds one block and whose last 256 columns hold 32, and

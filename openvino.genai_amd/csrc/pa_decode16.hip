@@ -349,15 +349,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void pa_decode16_kernel(Decod
     // ---- scores: the factors were formed in place of the block maxima before the merge --------------
     if (!a.want_scores) return;
     const float* fac = msnap;
-    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
     typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h4u __attribute__((ext_vector_type(4), aligned(2)));
     const long soff = st.score_offsets[b];
     if (final_out) {
-        // sum over the group's heads -> group_scores[hkv][position], four positions per thread;
-        // positions before the first block of the window get 0
-        float* dst = a.group_scores + (long)hkv * a.total_scores + soff;
+        // sum over the group's heads -> group_scores[hkv][position] (fp16, as in the u8 decode kernel), four positions
+        // per thread; positions before the first block of the window get 0
+        _Float16* dst = a.group_scores + (long)hkv * a.total_scores + soff;
         const int p0 = tb * TOK;
-        for (int pos = tid; pos < p0; pos += 64 * WAVES) dst[pos] = 0.0f;
+        for (int pos = tid; pos < p0; pos += 64 * WAVES) dst[pos] = (_Float16)0.0f;
         const int cnt = kv_len - p0;
         for (int lp = 4 * tid; lp < cnt; lp += 4 * 64 * WAVES) {
             const float* f = fac + (lp / TOK) * G;
@@ -371,9 +371,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void pa_decode16_kernel(Decod
                 sum[3] += (float)p4[3] * fh;
             }
             if (lp + 4 <= cnt) {
-                *reinterpret_cast<f4u*>(dst + p0 + lp) = sum;
+                *reinterpret_cast<h4u*>(dst + p0 + lp) = h4{(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
             } else {
-                for (int i = 0; lp + i < cnt; ++i) dst[p0 + lp + i] = sum[i];
+                for (int i = 0; lp + i < cnt; ++i) dst[p0 + lp + i] = (_Float16)sum[i];
             }
         }
     } else {

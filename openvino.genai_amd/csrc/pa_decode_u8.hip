@@ -468,15 +468,17 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 2) void pa_decode_u8_kern
     if (!a.want_scores) return;
     __syncthreads();
     const float* fac = msnap;
-    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
     typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h4u __attribute__((ext_vector_type(4), aligned(2)));
     const long soff = dsc->score_off;
     if (final_out) {
-        // sum over the group's heads -> group_scores[hkv][position], four positions per thread;
+        // sum over the group's heads -> group_scores[hkv][position], four positions per thread, handed on as fp16
+        // like the per-head probabilities of a launch with several splits (sums of at most 16 probabilities: the
+        // rounding is 2^-12 of the value, and half the bytes go to HBM and come back);
         // positions before the first block of the window get 0
-        float* dst = a.group_scores + (long)hkv * a.total_scores + soff;
+        _Float16* dst = a.group_scores + (long)hkv * a.total_scores + soff;
         const int p0 = tb * TOK;
-        for (int pos = tid; pos < p0; pos += NT) dst[pos] = 0.0f;
+        for (int pos = tid; pos < p0; pos += NT) dst[pos] = (_Float16)0.0f;
         const int cnt = kv_len - p0;
         for (int lp = 4 * tid; lp < cnt; lp += 4 * NT) {
             const float* f = fac + (lp / TOK) * 16;
@@ -490,9 +492,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 2) void pa_decode_u8_kern
                 sum[3] += (float)p4[3] * fh;
             }
             if (lp + 4 <= cnt) {
-                *reinterpret_cast<f4u*>(dst + p0 + lp) = sum;
+                *reinterpret_cast<h4u*>(dst + p0 + lp) = h4{(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
             } else {
-                for (int i = 0; lp + i < cnt; ++i) dst[p0 + lp + i] = sum[i];
+                for (int i = 0; lp + i < cnt; ++i) dst[p0 + lp + i] = (_Float16)sum[i];
             }
         }
     } else {
@@ -620,7 +622,7 @@ __device__ __forceinline__ void score_positions(const DecodeArgs& a, float* __re
             float s = 0.0f;
             if (live && pos >= first) {
 #pragma unroll 8
-                for (int h = 0; h < a.sh.Hkv; ++h) s += a.group_scores[(long)h * a.total_scores + soff + pos];
+                for (int h = 0; h < a.sh.Hkv; ++h) s += (float)a.group_scores[(long)h * a.total_scores + soff + pos];
             }
             scores[soff + pos] = s;
         }

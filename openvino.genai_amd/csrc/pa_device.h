@@ -256,7 +256,7 @@ struct DecodeArgs {
     float* part_acc;              // nsplit > 1: [T*Hq*nsplit, D] un-normalised
     float* part_ml;               // nsplit > 1: [T*Hq*nsplit, 2] (max in the log2 domain, denominator)
     float* final_ml;              // [T*Hq, 2]
-    float* group_scores;          // nsplit == 1: [Hkv, total_scores]
+    _Float16* group_scores;       // nsplit == 1: [Hkv, total_scores] per-kv-head score sums on their way to the score kernel
     _Float16* p_split;            // nsplit > 1: [Hq, p_split_stride(total_scores, B)] probabilities relative to the
                                   // split maximum; a sequence's run starts at p_split_offset (16-byte aligned)
 };

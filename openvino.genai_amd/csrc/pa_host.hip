@@ -741,8 +741,8 @@ void plan_items(pa_ctx* ctx) {
 // split probabilities): the context's growable buffers, or -- from_static -- pieces of the fixed device scratch, in
 // which case nothing is allocated and a step that needs more than the scratch holds is refused.
 struct DecodeWs {
-    float *part_acc, *part_ml, *final_ml, *group_scores;
-    _Float16* p_split;
+    float *part_acc, *part_ml, *final_ml;
+    _Float16 *group_scores, *p_split;
 };
 
 DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_scores, bool from_static) {
@@ -750,7 +750,7 @@ DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_sc
     const size_t b_final = rows * 2 * sizeof(float);
     const size_t b_acc = nsplit > 1 ? rows * nsplit * c.head_size * sizeof(float) : 0;
     const size_t b_ml = nsplit > 1 ? rows * nsplit * 2 * sizeof(float) : 0;
-    const size_t b_group = want_scores && nsplit == 1 ? (size_t)c.num_kv_heads * ctx->total_scores * sizeof(float) : 0;
+    const size_t b_group = want_scores && nsplit == 1 ? (size_t)c.num_kv_heads * ctx->total_scores * sizeof(uint16_t) : 0;
     const size_t b_psplit = want_scores && nsplit > 1
                                 ? (size_t)c.num_heads * pa::p_split_stride(ctx->total_scores, ctx->B) * sizeof(uint16_t) : 0;
     DecodeWs w{};
@@ -771,7 +771,7 @@ DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_sc
         w.final_ml = reinterpret_cast<float*>(base + o_final);
         w.part_acc = reinterpret_cast<float*>(base + o_acc);
         w.part_ml = reinterpret_cast<float*>(base + o_ml);
-        w.group_scores = reinterpret_cast<float*>(base + o_group);
+        w.group_scores = reinterpret_cast<_Float16*>(base + o_group);
         w.p_split = reinterpret_cast<_Float16*>(base + o_psplit);
         return w;
     }
@@ -783,7 +783,7 @@ DecodeWs decode_workspace(pa_ctx* ctx, size_t rows, int32_t nsplit, bool want_sc
     w.final_ml = ctx->final_ml.as<float>();
     w.part_acc = ctx->part_acc.as<float>();
     w.part_ml = ctx->part_ml.as<float>();
-    w.group_scores = ctx->group_scores.as<float>();
+    w.group_scores = ctx->group_scores.as<_Float16>();
     w.p_split = ctx->p_split.as<_Float16>();
     return w;
 }

@@ -73,7 +73,7 @@ def test_static_entry_point_refuses_what_it_cannot_serve(pkg):
     import torch
     from openvino_genai_amd import _lib as L
     dev = torch.device("cuda:0")
-    # more workspace than the scratch holds: per-kv-head score sums of 40 sequences x 30000 positions = 38 MB
+    # more workspace than the scratch holds: the per-head split probabilities of 40 sequences x 30000 positions, 77 MB
     op = pkg.PagedAttention(32, 8, 128, 32, "f16", "u8", 1, 0, torch.cuda.current_stream(dev))
     B, past = 40, 30000
     nblk = (past + 1 + 31) // 32

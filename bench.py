@@ -28,8 +28,8 @@ NUM_LAYERS_FOR_TOKS = 32  # Llama-3-8B depth: tok/s = batch / (32 * t_layer), at
 # WRITE_SIZE runs of it, scaled by the readings of a plain 1 GiB copy; the summary file holds commands and readings.
 # (a workload without a reading of the kernel as it stands is not listed: `traffic` is then null)
 MEASURED_TRAFFIC = {
-    "llama3_8b_decode_u8_b64_ctx4096": (585.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
-    "llama3_8b_eviction_u8_b256_ctx8192": (4656.2e6, "profiles/pa_decode_u8_kernel__llama3_8b_eviction_u8_b256_ctx8192.md"),
+    "llama3_8b_decode_u8_b64_ctx4096": (581.0e6, "profiles/pa_decode_u8_kernel__llama3_8b_decode_u8_b64_ctx4096.md"),
+    "llama3_8b_eviction_u8_b256_ctx8192": (4622.7e6, "profiles/pa_decode_u8_kernel__llama3_8b_eviction_u8_b256_ctx8192.md"),
     "long_context_decode_u8_b8_ctx32768": (594.4e6, "profiles/pa_decode_u8_kernel__long_context_decode_u8_b8_ctx32768.md"),
     "qwen25_7b_mixed_bf16": (218.8e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
 }

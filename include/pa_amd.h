@@ -150,7 +150,7 @@ typedef struct pa_layer_io {
  * kernels, correct but far from the tuned ones' speed.  In a step whose sequences all schedule one token, over a cache
  * the tuned kernels serve, the append is done by the attention kernel itself (the cache rows are the ones pa_kv_append
  * writes).  Head sizes 96 and 256 (K and V alike, the same caches) run on instantiations of the same kernels with
- * these limits: the matrix kernel keeps to 16 query rows per wave, block-sparse prefill is not offered, the u8 decode
+ * these limits: the matrix kernel keeps to 16 query rows per wave, block-sparse prefill is not offered at 96, the u8 decode
  * kernel does not take head size 256 with 16-token blocks (such steps run on the shape-generic kernel). */
 int32_t pa_forward(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* The op's `alibi_slopes` input (input 11: f32 [num_heads]; a graph constant that SDPAToPagedAttention leaves empty
@@ -271,7 +271,7 @@ float pa_xattention_threshold(float configured_threshold, uint64_t num_last_dens
  *     its groups; tokens outside the chunk count as zero vectors;
  *   - per (query head, I): key blocks 0 and I are kept, then the others in descending importance until the kept sum
  *     reaches threshold * the row's sum; a query row then sees a key position only if its block pair was kept.
- * Needs a cache block_size of 32, 64, 128 or 256, head_size 64 / 128 (K and V alike), a u8 cache or one of the query's
+ * Needs a cache block_size of 32, 64, 128 or 256, head_size 64 / 128 / 256 (K and V alike), a u8 cache or one of the query's
  * type; xattention_block_size a power of two >= 32, xattention_stride a power of two <= 32 (PA_NOT_IMPLEMENTED
  * otherwise). */
 int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t xattention_block_size,

@@ -1346,8 +1346,8 @@ int32_t pa_set_xattention(pa_ctx* ctx, const float* thresholds, int32_t block_si
             return;
         }
         PA_REQUIRE(!ctx->has_alibi, PA_NOT_IMPLEMENTED, "block-sparse prefill is not available with ALiBi slopes");
-        PA_REQUIRE(mfma_shape(c) && !narrow_only(c) && c.block_size >= 32, PA_NOT_IMPLEMENTED,
-                   "block-sparse prefill needs a block_size of 32 to 256 (a power of two), head_size 64 or 128 and a u8 cache "
+        PA_REQUIRE(mfma_shape(c) && c.head_size != 96 && c.block_size >= 32, PA_NOT_IMPLEMENTED,
+                   "block-sparse prefill needs a block_size of 32 to 256 (a power of two), head_size 64, 128 or 256 and a u8 cache "
                    "or one of the query's type");
         auto pow2 = [](int32_t v) { return v > 0 && (v & (v - 1)) == 0; };
         PA_REQUIRE(pow2(block_size) && block_size >= 32, PA_NOT_IMPLEMENTED,

@@ -435,13 +435,16 @@ hipError_t launch_xattention(hipStream_t s, const XattArgs& a, int q_dtype, int 
 #define PA_XLOGITS(DD, DT, Q, U8) \
     hipLaunchKernelGGL((xatt_logits_kernel<DD, DT, Q, U8>), lgrid, dim3(256), 0, s, a)
     const bool f16q = q_dtype == DT_F16;
-    if (a.sh.bs < 32 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1)) || (a.sh.D != 64 && a.sh.D != 128)) return hipErrorInvalidValue;
+    // (a stage is 64 channels of a slot: head sizes that are multiples of 64)
+    if (a.sh.bs < 32 || a.sh.bs > 256 || (a.sh.bs & (a.sh.bs - 1)) || (a.sh.D != 64 && a.sh.D != 128 && a.sh.D != 256)) return hipErrorInvalidValue;
     if (kv_dtype == DT_U8) {
         if (a.sh.D == 64) { if (f16q) PA_XLOGITS(64, DT_F16, DT_F16, true); else PA_XLOGITS(64, DT_F16, DT_BF16, true); }
-        else { if (f16q) PA_XLOGITS(128, DT_F16, DT_F16, true); else PA_XLOGITS(128, DT_F16, DT_BF16, true); }
+        else if (a.sh.D == 128) { if (f16q) PA_XLOGITS(128, DT_F16, DT_F16, true); else PA_XLOGITS(128, DT_F16, DT_BF16, true); }
+        else { if (f16q) PA_XLOGITS(256, DT_F16, DT_F16, true); else PA_XLOGITS(256, DT_F16, DT_BF16, true); }
     } else if (kv_dtype == q_dtype) {
         if (a.sh.D == 64) { if (f16q) PA_XLOGITS(64, DT_F16, DT_F16, false); else PA_XLOGITS(64, DT_BF16, DT_BF16, false); }
-        else { if (f16q) PA_XLOGITS(128, DT_F16, DT_F16, false); else PA_XLOGITS(128, DT_BF16, DT_BF16, false); }
+        else if (a.sh.D == 128) { if (f16q) PA_XLOGITS(128, DT_F16, DT_F16, false); else PA_XLOGITS(128, DT_BF16, DT_BF16, false); }
+        else { if (f16q) PA_XLOGITS(256, DT_F16, DT_F16, false); else PA_XLOGITS(256, DT_BF16, DT_BF16, false); }
     } else {
         return hipErrorInvalidValue;
     }

@@ -107,6 +107,9 @@ CASES = [
     ("stride_32", 8, 2, 128, "bf16", "bf16", [640], [384], 256, 32, 4.0),
     ("long_context_split", 8, 2, 128, "f16", "u8", [6000], [512], 64, 8, 4.0),
     ("gqa_7", 28, 4, 128, "bf16", "bf16", [2048], [512], 64, 8, 3.0),
+    # head size 256: four 64-channel stages per slot, the matrix kernel's one-row-group variant with one workgroup per CU
+    ("d256_f16", 8, 4, 256, "f16", "f16", [37, 1000], [300, 171], 64, 8, 4.0),
+    ("d256_u8_bf16", 16, 8, 256, "bf16", "u8", [100, 2500], [260, 333], 64, 8, 4.0),
 ]
 
 

@@ -208,9 +208,11 @@ hipError_t launch_ppl(hipStream_t s, uint8_t* kc, const Shape& sh, const int32_t
                       int32_t deltas_per_block, int32_t n, const float* lut) {
     const long rows = (long)n * sh.bs * sh.Hkv;
     const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-    if (sh.D > 128 || sh.D % 2) return hipErrorInvalidValue;
-    if (sh.D == 128 || sh.D == 64) {
-        if (sh.D == 128)
+    if ((sh.D > 128 && sh.D != 256) || sh.D % 2) return hipErrorInvalidValue;
+    if (sh.D == 256 || sh.D == 128 || sh.D == 64) {
+        if (sh.D == 256)
+            hipLaunchKernelGGL((pa_rotate_rows_kernel<KVDT, 16, 8>), dim3((unsigned)((rows + 31) / 32)), block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
+        else if (sh.D == 128)
             hipLaunchKernelGGL((pa_rotate_rows_kernel<KVDT, 8, 8>), dim3((unsigned)((rows + 31) / 32)), block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
         else
             hipLaunchKernelGGL((pa_rotate_rows_kernel<KVDT, 4, 8>), dim3((unsigned)((rows + 31) / 32)), block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);

@@ -230,7 +230,7 @@ int32_t pa_set_rotation_trig_lut(pa_ctx* ctx, const float* lut, int32_t rows);
  * (model_runner.hpp:1483-1509; deltas filled at pipeline_impl.cpp:856-872): re-rotates, in place, every K row of the
  * listed physical blocks of one layer's key cache (device pointer).  rotated_block_indices [n] and rotation_deltas
  * [n, deltas_per_block] (table rows; deltas_per_block is 1 or block_size) are host arrays.  Key caches of u8, f16
- * or bf16 rows with an even head size up to 128, or 256; other caches return PA_NOT_IMPLEMENTED. */
+ * or bf16 rows; u4 rows return PA_NOT_IMPLEMENTED. */
 int32_t pa_rotate_cache(pa_ctx* ctx, void* key_cache, int64_t num_blocks, const int32_t* rotated_block_indices,
                         int32_t num_rotated, const int32_t* rotation_deltas, int32_t deltas_per_block);
 

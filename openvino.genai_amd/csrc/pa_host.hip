@@ -1657,8 +1657,6 @@ int32_t pa_rotate_cache(pa_ctx* ctx, void* key_cache, int64_t num_blocks, const 
         PA_REQUIRE(key_cache && rotated_block_indices && rotation_deltas, PA_INVALID_C_PARAM, "null argument");
         PA_REQUIRE(ctx->trig_rows > 0, PA_NOT_ALLOCATED, "pa_set_rotation_trig_lut has not been called");
         PA_REQUIRE(c.kv_cache_dtype != PA_U4, PA_NOT_IMPLEMENTED, "cache rotation runs over u8, f16 and bf16 key caches");
-        PA_REQUIRE(c.head_size % 2 == 0 && (c.head_size <= 128 || c.head_size == 256), PA_NOT_IMPLEMENTED,
-                   "cache rotation runs for even head sizes up to 128, and 256");
         PA_REQUIRE(deltas_per_block == 1 || deltas_per_block == c.block_size, PA_PARAMETER_MISMATCH,
                    "rotation_deltas must hold 1 or block_size entries per block");
         for (int32_t i = 0; i < num_rotated; ++i)

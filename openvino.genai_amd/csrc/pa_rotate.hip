@@ -19,7 +19,7 @@
 namespace pa {
 namespace {
 
-// One pair per lane: head sizes up to 128 (with D = 64 the upper half of the wave idles).
+// A wave per row, PPL pairs per lane: head sizes up to 128 * PPL (lanes beyond half a row idle).
 template <int KVDT, int PPL>
 __global__ __launch_bounds__(256) void pa_rotate_kernel(uint8_t* __restrict__ key_cache, Shape sh,
                                                         const int32_t* __restrict__ rotated_block_indices,
@@ -208,7 +208,7 @@ hipError_t launch_ppl(hipStream_t s, uint8_t* kc, const Shape& sh, const int32_t
                       int32_t deltas_per_block, int32_t n, const float* lut) {
     const long rows = (long)n * sh.bs * sh.Hkv;
     const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-    if ((sh.D > 128 && sh.D != 256) || sh.D % 2) return hipErrorInvalidValue;
+    if (sh.D > 512 || sh.D % 8) return hipErrorInvalidValue;  // (half a row is a whole number of pairs per lane below)
     if (sh.D == 256 || sh.D == 128 || sh.D == 64) {
         if (sh.D == 256)
             hipLaunchKernelGGL((pa_rotate_rows_kernel<KVDT, 16, 8>), dim3((unsigned)((rows + 31) / 32)), block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
@@ -218,7 +218,9 @@ hipError_t launch_ppl(hipStream_t s, uint8_t* kc, const Shape& sh, const int32_t
             hipLaunchKernelGGL((pa_rotate_rows_kernel<KVDT, 4, 8>), dim3((unsigned)((rows + 31) / 32)), block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((pa_rotate_kernel<KVDT, 1>), grid, block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
+    if (sh.D <= 128) hipLaunchKernelGGL((pa_rotate_kernel<KVDT, 1>), grid, block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
+    else if (sh.D <= 256) hipLaunchKernelGGL((pa_rotate_kernel<KVDT, 2>), grid, block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
+    else hipLaunchKernelGGL((pa_rotate_kernel<KVDT, 4>), grid, block, 0, s, kc, sh, idx, deltas, deltas_per_block, n, lut);
     return hipGetLastError();
 }
 

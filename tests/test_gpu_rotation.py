@@ -27,7 +27,8 @@ def _random_cache(rng, nb, Hkv, bs, D, kd):
 
 @pytest.mark.parametrize("kd,D,per_token", [("u8", 128, False), ("u8", 64, True), ("f16", 128, False), ("bf16", 64, False),
                                             ("f16", 64, True), ("bf16", 128, True), ("u8", 256, True), ("bf16", 256, False),
-                                            ("u8", 96, False), ("f16", 96, True)])
+                                            ("u8", 96, False), ("f16", 96, True), ("u8", 192, True), ("bf16", 512, False),
+                                            ("u8", 80, False)])
 def test_rotate_cache_bit_exact(pkg, dev, kd, D, per_token):
     import torch
     print(f"case rotate {kd} D={D} per_token={per_token}", flush=True)

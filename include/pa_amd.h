@@ -425,8 +425,9 @@ int32_t pa_evictor_block_scores(pa_evictor* ev, int32_t slot, int32_t layer, dou
  * sum, over the rows of a block, of the head-averaged cosine similarities that are not below their
  * row's mean.  The matrices are concatenated in `diversity` (device, `capacity` floats);
  * offsets[b] .. offsets[b+1] (host, B + 1 entries, may be NULL) is sequence b's span.  Uses the
- * block table of `layer` set by pa_set_block_indices in this step; block size 32, head size 64, 96,
- * 128 or 256.  `evictable_sizes` is a HOST array of B entries.  The optional block-set inputs
+ * block table of `layer` set by pa_set_block_indices in this step.  Block size 32 with head size 64, 96, 128 or 256
+ * over u8 / f16 / bf16 keys runs on the matrix cores, every other shape pa_create accepts on the vector unit (the
+ * same values, far slower).  `evictable_sizes` is a HOST array of B entries.  The optional block-set inputs
  * (`adaptive_rkv_diversity_block_set_indices.<L>`, model_runner.hpp:1691-1770) only permit computing
  * less; every block is computed here.
  * The arithmetic of this output lives in OpenVINO (2026.4 development line, the reference's pinned

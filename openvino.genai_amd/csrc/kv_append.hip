@@ -19,7 +19,6 @@ constexpr int TOKENS_KERNEL_MIN_T = 8192;  // steps of this many tokens take the
 template <int QDT, int KVDT, int E>
 __device__ __forceinline__ void append_row(uint32_t (&w)[E / 2], uint8_t* dst, int l16) {
 #pragma clang fp contract(off)
-    constexpr int D = 16 * E;
     if constexpr (KVDT == DT_U8) {
         float x[E];
 #pragma unroll

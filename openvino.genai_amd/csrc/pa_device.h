@@ -655,9 +655,9 @@ hipError_t launch_scores_replay(hipStream_t s, const StepDev& st, const Shape& s
 struct RkvDivSeq {          // one sequence whose diversity is computed
     int32_t table_off;      // first entry of the sequence's block table
     int32_t first_block;    // logical block the evictable area starts at
-    int32_t ev;             // evictable tokens, a multiple of 32
+    int32_t ev;             // evictable tokens, a multiple of the block size
     int32_t tok_off;        // first entry of the sequence in the per-token arrays (per head: + h * total_tok)
-    int64_t out_off;        // first output value: [ev / 32, ev] floats
+    int64_t out_off;        // first output value: [ev / block size, ev] floats
 };
 struct RkvDivArgs {
     const uint8_t* key_cache;
@@ -673,5 +673,8 @@ struct RkvDivArgs {
 };
 int rkv_diversity_chunks(int ev_max);
 hipError_t launch_rkv_diversity(hipStream_t s, const RkvDivArgs& a, int kv_dtype, int D, int bs, int nseq, int ev_max);
+// The same output for any head size that is a multiple of 8, any block size and u4 rows too, on
+// the vector unit (pa_generic.hip); the column sums are kept per chunk of 256 tokens, as rkv_diversity_chunks counts.
+hipError_t launch_rkv_diversity_generic(hipStream_t s, const RkvDivArgs& a, int kv_dtype, int D, int bs, int nseq, int ev_max);
 
 }  // namespace pa

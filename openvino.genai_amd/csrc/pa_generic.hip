@@ -505,6 +505,178 @@ hipError_t launch_attention_generic(hipStream_t s, const StepDev& st, const Gene
     return hipErrorInvalidValue;
 }
 
+// ---- block diversity for every shape (what pa_rkv_diversity.hip does on the matrix cores for its shapes) ----------
+// out[block][c] = -(1 / Hkv) * sum over kv heads and over the block's rows r of cos(k_r, k_c), with the diagonal set
+// to zero and entries below their row's mean (over the whole area) dropped.  Three passes over the area's key rows,
+// every sum in a fixed order:
+//   1. per token: 1 / |k| -> `stats[..].x` (and k^ . k^ -> .w); per chunk of 256 tokens the column sums of k^ -> `colsum`;
+//   2. per token: the row's mean -> `mean`, from k^_r . (sum over the area of k^) - k^_r . k^_r;
+//   3. per (block, 64 columns): the similarities, 16 rows of k^ at a time through LDS.
+namespace {
+constexpr int GDIV_CHUNK = 256;
+constexpr float GDIV_EPS = 1e-12f;
+
+// The lane's eight channels (8 lane ..) of token j of the area, as floats; lanes beyond the row get zeros.
+__device__ __forceinline__ void gdiv_load(const RkvDivArgs& a, const RkvDivSeq& q, const int32_t* table, int h, int j,
+                                          int D, int bs, int dt, int lane, float (&x)[8]) {
+    const int pos = q.first_block * bs + j;
+    RowReader rr(a.key_cache, table[pos / bs], h, pos % bs, a.Hkv, bs, D, dt);
+    if (8 * lane < D) {
+        rr.load8(8 * lane, x);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0.0f;
+    }
+}
+
+__global__ __launch_bounds__(256) void gdiv_norm_colsum_kernel(RkvDivArgs a, int D, int bs, int dt) {
+    __shared__ float red[4][MAX_D];
+    const RkvDivSeq q = a.seqs[blockIdx.z];
+    const int h = blockIdx.y, base = blockIdx.x * GDIV_CHUNK;
+    if (base >= q.ev) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int32_t* table = a.block_indices + q.table_off;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    for (int j = base + wv; j < min(base + GDIV_CHUNK, q.ev); j += 4) {  // (wave-uniform bounds)
+        float x[8];
+        gdiv_load(a, q, table, h, j, D, bs, dt, lane, x);
+        float sq = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq = fmaf(x[e], x[e], sq);
+        sq = wave_sum(sq);
+        const float inv = 1.0f / sqrtf(sq + GDIV_EPS);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(x[e], inv, acc[e]);
+        if (lane == 0) a.stats[(long)h * a.total_tok + q.tok_off + j] = make_float4(inv, 0.0f, 0.0f, sq * inv * inv);
+    }
+    if (8 * lane < D) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[wv][8 * lane + e] = acc[e];
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += 256)
+        a.colsum[(((long)blockIdx.z * a.Hkv + h) * (a.chunks_max + 1) + 1 + blockIdx.x) * D + d] =
+            ((red[0][d] + red[1][d]) + red[2][d]) + red[3][d];
+}
+
+__global__ __launch_bounds__(256) void gdiv_total_kernel(RkvDivArgs a, int D) {
+    const RkvDivSeq q = a.seqs[blockIdx.y];
+    const int chunks = (q.ev + GDIV_CHUNK - 1) / GDIV_CHUNK;
+    float* cs = a.colsum + ((long)blockIdx.y * a.Hkv + blockIdx.x) * (a.chunks_max + 1) * D;
+    for (int d = threadIdx.x; d < D; d += 256) {
+        float s = 0.0f;
+        for (int c = 0; c < chunks; ++c) s += cs[(long)(1 + c) * D + d];
+        cs[d] = s;
+    }
+}
+
+__global__ __launch_bounds__(256) void gdiv_mean_kernel(RkvDivArgs a, int D, int bs, int dt) {
+    const RkvDivSeq q = a.seqs[blockIdx.z];
+    const int h = blockIdx.y;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int j = blockIdx.x * 4 + wv;
+    if (j >= q.ev) return;  // (wave-uniform)
+    const int32_t* table = a.block_indices + q.table_off;
+    const float* tot = a.colsum + ((long)blockIdx.z * a.Hkv + h) * (a.chunks_max + 1) * D;
+    float x[8];
+    gdiv_load(a, q, table, h, j, D, bs, dt, lane, x);
+    float d = 0.0f;
+    if (8 * lane < D) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(x[e], tot[8 * lane + e], d);
+    }
+    d = wave_sum(d);
+    const float4 st = a.stats[(long)h * a.total_tok + q.tok_off + j];
+    if (lane == 0) a.mean[(long)h * a.total_tok + q.tok_off + j] = (d * st.x - st.w) / (float)q.ev;
+}
+
+// A workgroup = one block of rows x 64 columns: thread (column c of the 64, quarter qd) holds its column's row of one
+// kv head in registers, D elements at most 128 at a time, and meets rows 4 * i + qd of every 16-row slice of the block
+// in LDS.
+__global__ __launch_bounds__(256) void gdiv_pair_kernel(RkvDivArgs a, int D, int bs, int dt) {
+    __shared__ __align__(16) float rows[16][128 + 4];
+    __shared__ float rmean[16], part[4][64];
+    const RkvDivSeq q = a.seqs[blockIdx.z];
+    const int rb = blockIdx.y;
+    if (rb * bs >= q.ev || (int)blockIdx.x * 64 >= q.ev) return;
+    const int cl = threadIdx.x & 63, qd = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cl;
+    const bool col_ok = c < q.ev;
+    const int cj = min(c, q.ev - 1);
+    const int32_t* table = a.block_indices + q.table_off;
+    float total = 0.0f;
+    for (int h = 0; h < a.Hkv; ++h) {
+        const long sbase = (long)h * a.total_tok + q.tok_off;
+        const float c_inv = a.stats[sbase + cj].x;
+        const int cpos = q.first_block * bs + cj;
+        RowReader cr(a.key_cache, table[cpos / bs], h, cpos % bs, a.Hkv, bs, D, dt);
+        const int rend = (rb + 1) * bs;
+        for (int r0 = rb * bs; r0 < rend; r0 += 16) {  // (a last slice may hold fewer than 16 rows: the others are zeros that count for nothing)
+            float dot[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int d0 = 0; d0 < D; d0 += 128) {
+                const int dn = min(128, D - d0);
+                __syncthreads();  // the slice staged before is done with
+                // stage rows r0 .. r0 + 15, channels d0 .. d0 + dn - 1, as k^ (thread t: row t / 16, eight channels)
+                {
+                    const int rr_ = threadIdx.x >> 4, ch = (threadIdx.x & 15) * 8;
+                    if (ch < dn) {
+                        const int rj = min(r0 + rr_, rend - 1);
+                        const int rpos = q.first_block * bs + rj;
+                        RowReader rr(a.key_cache, table[rpos / bs], h, rpos % bs, a.Hkv, bs, D, dt);
+                        float x[8];
+                        rr.load8(d0 + ch, x);
+                        const float inv = r0 + rr_ < rend ? a.stats[sbase + rj].x : 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) rows[rr_][ch + e] = x[e] * inv;
+                    }
+                    if (d0 == 0 && threadIdx.x < 16)
+                        rmean[threadIdx.x] = r0 + (int)threadIdx.x < rend ? a.mean[sbase + r0 + threadIdx.x] : INFINITY;
+                }
+                __syncthreads();
+                for (int d = 0; d < dn; d += 8) {
+                    float y[8];
+                    cr.load8(d0 + d, y);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 ra = *reinterpret_cast<const float4*>(&rows[4 * i + qd][d]);
+                        const float4 rb4 = *reinterpret_cast<const float4*>(&rows[4 * i + qd][d + 4]);
+                        dot[i] = fmaf(y[0], ra.x, dot[i]); dot[i] = fmaf(y[1], ra.y, dot[i]);
+                        dot[i] = fmaf(y[2], ra.z, dot[i]); dot[i] = fmaf(y[3], ra.w, dot[i]);
+                        dot[i] = fmaf(y[4], rb4.x, dot[i]); dot[i] = fmaf(y[5], rb4.y, dot[i]);
+                        dot[i] = fmaf(y[6], rb4.z, dot[i]); dot[i] = fmaf(y[7], rb4.w, dot[i]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = r0 + 4 * i + qd;
+                const float v = r == c ? 0.0f : dot[i] * c_inv;
+                total += v < rmean[4 * i + qd] ? 0.0f : v;
+            }
+        }
+    }
+    __syncthreads();
+    part[qd][cl] = total;
+    __syncthreads();
+    if (qd == 0 && col_ok)
+        a.out[q.out_off + (long)rb * q.ev + c] = -((((part[0][cl] + part[1][cl]) + part[2][cl]) + part[3][cl]) / (float)a.Hkv);
+}
+}  // namespace
+
+hipError_t launch_rkv_diversity_generic(hipStream_t s, const RkvDivArgs& a, int kv_dtype, int D, int bs, int nseq, int ev_max) {
+    if (nseq == 0 || ev_max == 0) return hipSuccess;
+    if (D <= 0 || D > MAX_D || D % 8 || bs <= 0 || ev_max % bs) return hipErrorInvalidValue;
+    const int chunks = (ev_max + GDIV_CHUNK - 1) / GDIV_CHUNK;
+    if (chunks > a.chunks_max) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gdiv_norm_colsum_kernel, dim3((unsigned)chunks, (unsigned)a.Hkv, (unsigned)nseq), dim3(256), 0, s, a, D, bs, kv_dtype);
+    hipLaunchKernelGGL(gdiv_total_kernel, dim3((unsigned)a.Hkv, (unsigned)nseq), dim3(256), 0, s, a, D);
+    hipLaunchKernelGGL(gdiv_mean_kernel, dim3((unsigned)((ev_max + 3) / 4), (unsigned)a.Hkv, (unsigned)nseq), dim3(256), 0, s, a, D, bs, kv_dtype);
+    hipLaunchKernelGGL(gdiv_pair_kernel, dim3((unsigned)((ev_max + 63) / 64), (unsigned)(ev_max / bs), (unsigned)nseq), dim3(256), 0, s, a, D, bs, kv_dtype);
+    return hipGetLastError();
+}
+
 hipError_t launch_kv_append_generic(hipStream_t s, const StepDev& st, const GenericShape& sh, int q_dtype, const void* key,
                                     const void* value, void* key_cache, void* value_cache, const int32_t* block_indices) {
     if (!generic_shape_ok(sh)) return hipErrorInvalidValue;

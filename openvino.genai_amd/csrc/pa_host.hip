@@ -1688,8 +1688,9 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         PA_REQUIRE(ctx->step_ready, PA_PARAMETER_MISMATCH, "pa_step_begin has not been called");
         PA_REQUIRE(evictable_sizes, PA_INVALID_C_PARAM, "adaptive_rkv_evictable_sizes missing");
         PA_REQUIRE(layer >= 0 && layer < c.num_layers, PA_OUT_OF_BOUNDS, "layer out of range");
-        PA_REQUIRE(c.block_size == 32 && (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || c.head_size == 256) && c.kv_cache_dtype != PA_U4, PA_NOT_IMPLEMENTED,
-                   "block diversity runs for block size 32, head size 64, 96, 128 or 256 and a u8, f16 or bf16 key cache");
+        // the matrix-core kernels' shapes; everything else runs on the vector unit
+        const bool tuned = c.block_size == 32 && (c.head_size == 64 || c.head_size == 96 || c.head_size == 128 || c.head_size == 256) &&
+                           c.kv_cache_dtype != PA_U4;
         PA_REQUIRE(start_size >= 0 && start_size % c.block_size == 0, PA_PARAMETER_MISMATCH,
                    "adaptive_rkv_start_size must be a non-negative multiple of the block size");
         const size_t tidx = ctx->shared_table ? 0 : (size_t)layer;
@@ -1744,7 +1745,10 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         a.Hkv = c.num_kv_heads;
         a.total_tok = (int32_t)tok_total;
         a.chunks_max = chunks;
-        HIP_CHECK(pa::launch_rkv_diversity(ctx->stream, a, c.kv_cache_dtype, c.head_size, c.block_size, (int)seqs.size(), ev_max));
+        if (tuned)
+            HIP_CHECK(pa::launch_rkv_diversity(ctx->stream, a, c.kv_cache_dtype, c.head_size, c.block_size, (int)seqs.size(), ev_max));
+        else
+            HIP_CHECK(pa::launch_rkv_diversity_generic(ctx->stream, a, c.kv_cache_dtype, c.head_size, c.block_size, (int)seqs.size(), ev_max));
     });
 }
 

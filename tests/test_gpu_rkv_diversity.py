@@ -1,5 +1,5 @@
-"""Block diversity of the evictable area on the GPU (matrix cores) against the CPU checker on the same paged key
-caches.  Tolerance 2e-3 relative / 1e-3 absolute, plus the checker's own slack for similarities that sit within
+"""Block diversity of the evictable area on the GPU (matrix cores; the vector unit for shapes the matrix-core kernels
+are not built for) against the CPU checker on the same paged key caches.  Tolerance 2e-3 relative / 1e-3 absolute, plus the checker's own slack for similarities that sit within
 2e-5 of their row's mean (dropping entries below the mean is a step function: a value computed in f32 may fall on
 the other side of it)."""
 import numpy as np
@@ -12,11 +12,10 @@ pytestmark = pytest.mark.gpu
 RTOL, ATOL, MARGIN = 2e-3, 1e-3, 2e-5
 
 
-def _run(pkg, kv, q, Hq, Hkv, D, lens, start, ev_sizes, seed, keys=None):
+def _run(pkg, kv, q, Hq, Hkv, D, lens, start, ev_sizes, seed, keys=None, bs=32):
     import torch
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(seed)
-    bs = 32
     kc, ids, bib = RC.paged_key_cache(rng, lens, Hkv, D, bs, kv, q, keys=keys)
     B = len(lens)
     op = pkg.PagedAttention(Hq, Hkv, D, bs, q, kv, num_layers=2, device=0, stream=torch.cuda.current_stream(dev))
@@ -60,6 +59,17 @@ def test_diversity_matches_checker(pkg, kv, q, D):
     got, res = _run(pkg, kv, q, 8, 2, D, lens, 64, ev, seed=D + len(kv))
     assert len(res) == 4
     assert max(np.abs(r).max() for _, r in res) > 1.0
+
+
+@pytest.mark.parametrize("kv,q,D,bs", [("u8", "f16", 80, 32), ("f16", "f16", 128, 16), ("bf16", "bf16", 64, 24), ("u8", "bf16", 192, 64),
+                                       ("f16", "f16", 512, 16), ("u8", "f16", 128, 128), ("u8", "f16", 8, 32)])
+def test_diversity_of_other_shapes(pkg, kv, q, D, bs):
+    """Head sizes and block sizes the matrix-core kernels are not built for: the same output from the vector unit."""
+    lens = [25 * bs + 7, 9 * bs + 1, 40, 3 * bs]
+    ev = [20 * bs, 7 * bs, 0, bs]
+    got, res = _run(pkg, kv, q, 8, 2, D, lens, 2 * bs, ev, seed=D + bs, bs=bs)
+    assert len(res) == 3
+    assert max(np.abs(r).max() for _, r in res) > 0.5
 
 
 @pytest.mark.parametrize("kv,q,D", [("u8", "f16", 128), ("bf16", "bf16", 64), ("f16", "f16", 128), ("u8", "bf16", 96),

@@ -40,7 +40,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, help="workload (2 = headline; 1, 4, 5 and -- other head sizes -- 6, 7 for diagnostics)")
+    ap.add_argument("--config", type=int, default=2, help="workload (2 = headline; 1, 4, 5, other head sizes 6, 7 and larger prefill steps 8, 9 for diagnostics)")
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--sliding-window", type=int, default=None)
     ap.add_argument("--block-size", type=int, choices=[16, 32], default=None,

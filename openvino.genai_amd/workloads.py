@@ -28,11 +28,17 @@ CONFIGS = {
             past=("const", 4096), new=1, sliding_window=0),
     7: dict(name="gemma2_9b_decode_u8_b64_ctx4096", Hq=16, Hkv=8, D=256, bs=32, q_dtype="f16", kv_dtype="u8", B=64,
             past=("const", 4096), new=1, sliding_window=0),
+    # ... and larger prefill steps than the mixed workload's four 512-token chunks (Qwen2.5-7B shape, bf16): one
+    # 2048-token chunk behind 30000 cached tokens, and an 8192-token prompt from scratch
+    8: dict(name="qwen25_7b_prefill_bf16_2048_behind_30000", Hq=28, Hkv=4, D=128, bs=32, q_dtype="bf16", kv_dtype="bf16",
+            B=1, past=("mixed", [30000], 0, 1, 1), new=("mixed", 2048, 1), sliding_window=0),
+    9: dict(name="qwen25_7b_prefill_bf16_8192_from_scratch", Hq=28, Hkv=4, D=128, bs=32, q_dtype="bf16", kv_dtype="bf16",
+            B=1, past=("mixed", [0], 0, 1, 1), new=("mixed", 8192, 1), sliding_window=0),
 }
 
 
 def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0, block_size=None):
-    """Step metadata of config ``cfg`` (1..7); ``batch`` / ``context_scale`` shrink it for parity tests."""
+    """Step metadata of config ``cfg`` (1..9); ``batch`` / ``context_scale`` shrink it for parity tests."""
     c = dict(CONFIGS[cfg])
     rng = np.random.Generator(np.random.PCG64(1000 + cfg if seed is None else seed))
     B = c["B"] if batch is None else batch

@@ -32,6 +32,8 @@ MEASURED_TRAFFIC = {
     "llama3_8b_eviction_u8_b256_ctx8192": (4622.7e6, "profiles/pa_decode_u8_kernel__llama3_8b_eviction_u8_b256_ctx8192.md"),
     "long_context_decode_u8_b8_ctx32768": (594.4e6, "profiles/pa_decode_u8_kernel__long_context_decode_u8_b8_ctx32768.md"),
     "qwen25_7b_mixed_bf16": (218.8e6, "profiles/pa_prefill16_kernel__qwen25_7b_mixed_bf16.md"),
+    "phi3_mini_decode_u8_b64_ctx4096": (1777.6e6, "profiles/pa_decode_kernels__head_sizes_96_256_decode_b64_ctx4096.md"),
+    "gemma2_9b_decode_u8_b64_ctx4096": (1122.3e6, "profiles/pa_decode_kernels__head_sizes_96_256_decode_b64_ctx4096.md"),
 }
 
 

@@ -536,6 +536,15 @@ def test_fused_append_row_is_seen_by_the_launch_that_writes_it(pkg, dev, qd, kd,
 
 
 
+@pytest.mark.parametrize("qd,kd,new", [("f16", "u8", [1, 1]), ("bf16", "bf16", [1, 1]), ("f16", "u8", [1, 300]), ("bf16", "bf16", [1, 300])])
+def test_contexts_of_128k_tokens(pkg, dev, qd, kd, new):
+    """Two sequences behind 131071 and 70000 cached tokens, decoding or with a chunk beside the long one: the split
+    plans at their limits (64 splits, the most tiles a workgroup's LDS holds), int32 offsets far from their ends."""
+    case = H.case_from_lens(f"ctx128k_{qd}_{kd}_{new[1]}", 8, 2, 128, 32, qd, kd, [131071, 70000], new,
+                            score_aggregation_window=[1, min(new[1], 4)])
+    _check(pkg, dev, case, 99)
+
+
 def test_decode_u8_ignores_garbage_beyond_the_context(pkg, dev):
     """Rows past kv_len in the last block (and unused blocks) may hold anything, NaN headers included."""
     case = H.case_from_lens("garbage_tail", 8, 2, 128, 32, "f16", "u8", [40, 90], [1, 1])

@@ -545,6 +545,18 @@ def test_contexts_of_128k_tokens(pkg, dev, qd, kd, new):
     _check(pkg, dev, case, 99)
 
 
+@pytest.mark.parametrize("qd,kd,mixed", [("f16", "u8", False), ("bf16", "bf16", False), ("f16", "u8", True), ("f16", "f16", True)])
+def test_steps_of_three_thousand_sequences(pkg, dev, qd, kd, mixed):
+    """Many short sequences in one step (grids, descriptors and lists far beyond the benchmark's batch sizes), all
+    decoding or every seventh one with a short chunk."""
+    rng = np.random.default_rng(5)
+    B = 3000
+    past = rng.integers(0, 120, B).tolist()
+    new = [int(rng.integers(2, 40)) if mixed and i % 7 == 0 else 1 for i in range(B)]
+    case = H.case_from_lens(f"many_seqs_{qd}_{kd}_{mixed}", 8, 2, 64, 32, qd, kd, past, new)
+    _check(pkg, dev, case, 17)
+
+
 def test_decode_u8_ignores_garbage_beyond_the_context(pkg, dev):
     """Rows past kv_len in the last block (and unused blocks) may hold anything, NaN headers included."""
     case = H.case_from_lens("garbage_tail", 8, 2, 128, 32, "f16", "u8", [40, 90], [1, 1])

@@ -13,6 +13,11 @@
  * Pointer spaces: `*_dev` / tensors named like the op's inputs live in device memory (HBM);
  * the small int32 step arrays are HOST pointers -- they are what ModelRunner::forward fills on
  * the host each step -- and are uploaded once per step by pa_step_begin.
+ *
+ * Threads: the library keeps no state outside its handles.  Different handles may be used by different
+ * host threads at the same time (the reference drives one pipeline per thread); the calls on ONE handle
+ * must not overlap.  `pa_global_last_error` is per thread.  The one exception is pa_attention_static,
+ * whose calls on one GPU share that GPU's scratch array whatever handle they are made on.
  */
 #ifndef PA_AMD_H
 #define PA_AMD_H

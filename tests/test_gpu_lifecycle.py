@@ -86,3 +86,41 @@ def test_contexts_of_different_shapes_used_in_turn_give_the_bits_they_give_alone
                 assert np.array_equal(again[what], alone[i][what], equal_nan=what == "scores"), (rnd, cases[i]["name"], what)
     want = H.run_case_on_checker(cases[0])
     H.assert_close(alone[0]["out"], want["out"], cases[0]["q_dtype"])
+
+
+def test_two_host_threads_each_with_contexts_and_a_stream_of_their_own(pkg):
+    """The library keeps no state outside its handles (error texts of handle-less calls are per thread): two host
+    threads that create, use and destroy contexts at the same time, each on its own stream, get the bits a single
+    thread gets."""
+    import threading
+    import torch
+    dev = torch.device("cuda:0")
+    cases = _cases()
+    alone = [H.run_case_on_gpu(pkg, c, dev) for c in cases]
+    for a in alone:
+        a["op"] = None
+    problems = []
+
+    def worker(k):
+        try:
+            s = torch.cuda.Stream(dev)
+            with torch.cuda.stream(s):
+                for rep in range(5):
+                    order = list(range(len(cases)))
+                    if k:
+                        order.reverse()
+                    for i in order:
+                        r = H.run_case_on_gpu(pkg, cases[i], dev)
+                        for what in ("out16", "scores", "key_cache", "value_cache"):
+                            if not np.array_equal(r[what], alone[i][what]):
+                                problems.append((k, rep, cases[i]["name"], what))
+                        r["op"] = None
+        except BaseException as e:  # noqa: BLE001 -- reported by the main thread
+            problems.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not problems, problems[:5]

@@ -178,7 +178,7 @@ int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
  * 16 query heads per kv head); other steps return
  * PA_NOT_IMPLEMENTED.  The split partials,
  * final maxima / denominators and the score staging live in a fixed device array of PA_STATIC_SCRATCH_BYTES bytes
- * (32 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls
+ * (40 MiB; one per GPU, held until the process ends) instead of the context's growable buffers: the call itself calls
  * no hipMalloc / hipFree, and the device code of its kernels is uploaded by pa_create, not by the first call (the
  * runtime would otherwise allocate for it inside that call); a step that needs more returns PA_OUT_OF_BOUNDS and a
  * message with the byte count.  (The
@@ -186,7 +186,7 @@ int32_t pa_attention(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
  * as for pa_attention.)  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race, also from
  * different contexts; calls in stream order on one stream do not.  Nothing in it needs clearing between calls: each
  * call writes every element it later reads. */
-#define PA_STATIC_SCRATCH_BYTES (32u << 20)
+#define PA_STATIC_SCRATCH_BYTES (40u << 20)
 int32_t pa_attention_static(pa_ctx* ctx, int32_t layer, const pa_layer_io* io);
 /* Blocks until everything launched on the context's stream has finished. */
 int32_t pa_synchronize(pa_ctx* ctx);

@@ -11,7 +11,7 @@ SO_PATH = os.environ.get("PA_AMD_LIBRARY") or os.path.join(_HERE, "csrc", "libpa
 
 PA_OK = 0
 PA_F16, PA_BF16, PA_U8, PA_U4 = 0, 1, 2, 3
-PA_STATIC_SCRATCH_BYTES = 32 << 20
+PA_STATIC_SCRATCH_BYTES = 40 << 20
 PA_AGG_SUM, PA_AGG_NORM_SUM, PA_AGG_ADAPTIVE_RKV = 0, 1, 2
 (PA_KVCRUSH_ANCHOR_RANDOM, PA_KVCRUSH_ANCHOR_ZEROS, PA_KVCRUSH_ANCHOR_ONES, PA_KVCRUSH_ANCHOR_MEAN,
  PA_KVCRUSH_ANCHOR_ALTERNATING) = range(5)

@@ -95,3 +95,34 @@ def test_static_entry_point_refuses_what_it_cannot_serve(pkg):
     with pytest.raises(L.PaError) as e:
         op.attention_static(q, kc, kc, out, None)
     assert e.value.status == -2
+
+
+def test_static_entry_point_serves_the_largest_single_token_workload(pkg):
+    """256 sequences x 8193 positions, 32 heads over 8 kv heads: the per-kv-head score sums alone are 33.6 MB, the
+    largest workspace among the single-token workloads this path is measured on, and inside the scratch.  The block
+    tables walk a pool of 129 real blocks over and over, so the case costs megabytes, not gigabytes."""
+    import torch
+    from oracle import oracle as O
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D, bs, B, ctx_len = 32, 8, 128, 32, 256, 8193
+    pool = H.build_case(H.case_from_lens("static_pool", Hq, Hkv, D, bs, "f16", "u8", [4095], [1]), seed=21, pool_factor=1.0)
+    nb, nblk = pool["num_blocks"], (ctx_len + bs - 1) // bs
+    rng = np.random.default_rng(22)
+    case = dict(pool, name="static_256x8193", B=B, past_lens=np.full(B, ctx_len - 1, np.int32), new_lens=np.ones(B, np.int32),
+                subsequence_begins=np.arange(B + 1, dtype=np.int32),
+                block_indices_begins=(np.arange(B + 1) * nblk).astype(np.int32),
+                block_indices=rng.integers(0, nb, B * nblk).astype(np.int32),
+                query=O.to_bits(rng.standard_normal((B, Hq * D)).astype(np.float32), H.DT["f16"]))
+    ref_op = pkg.PagedAttention(Hq, Hkv, D, bs, "f16", "u8", 1, 0, torch.cuda.current_stream(dev))
+    st_op = pkg.PagedAttention(Hq, Hkv, D, bs, "f16", "u8", 1, 0, torch.cuda.current_stream(dev))
+    out_s, sc_s, ns = _run(torch, st_op, case, dev, static=True)
+    out_r, sc_r, nr = _run(torch, ref_op, case, dev, static=False)
+    assert ns == nr == 1
+    assert Hkv * sc_s.size * 2 > 32 << 20
+    assert np.array_equal(out_s, out_r)
+    assert np.array_equal(sc_s, sc_r)
+    out, out16, scores = O.paged_attention(case["query"], H.DT["f16"], case["key_cache0"], case["value_cache0"], H.DT["u8"],
+                                           case["past_lens"], case["subsequence_begins"], case["block_indices"],
+                                           case["block_indices_begins"], Hq, Hkv, D, bs, case["scale"], 0, None, True, 8)
+    H.assert_close(O.from_bits(out_s, H.DT["f16"]), out, "f16")
+    H.assert_close(sc_s, scores, "f16", "scores")

@@ -302,7 +302,9 @@ def test_full_size_scoring_workload_eviction_matches_checker(pkg, snapkv):
         caches.append(pair)
     perm = rng.permutation(pool)
     tables = [[list(perm[b * (nblk0 + 1): b * (nblk0 + 1) + nblk0]) for b in range(B)] for _ in range(L)]
-    spare = [[int(perm[b * (nblk0 + 1) + nblk0])] for b in range(B)]   # one more block per sequence, for growth
+    # one more block per sequence and layer, for growth; like the reference's allocator, every layer has a free list
+    # of its own (a block freed by layer l's eviction is only ever handed back to layer l)
+    spare = [[[int(perm[b * (nblk0 + 1) + nblk0])] for b in range(B)] for _ in range(L)]
     cfg = pkg.CacheEvictionConfig(start, recent, mx, pkg.AggregationMode.NORM_SUM, False, snapkv)
     ev = pkg.Evictor(cfg, bs, L, 7, max_sequences=B, max_tracked_tokens=ctx0 + 64, device=0,
                      stream=torch.cuda.current_stream(dev))
@@ -315,9 +317,8 @@ def test_full_size_scoring_workload_eviction_matches_checker(pkg, snapkv):
     for step in range(34):
         for b in range(B):
             if (past[b] + 1 + bs - 1) // bs > len(tables[0][b]):
-                blk = spare[b].pop()
                 for l in range(L):
-                    tables[l][b].append(blk)
+                    tables[l][b].append(spare[l][b].pop())
         q = torch.randn(B, Hq * D, device=dev, generator=gen).to(torch.float16)
         k = torch.randn(B, Hkv * D, device=dev, generator=gen).to(torch.float16)
         v = torch.randn(B, Hkv * D, device=dev, generator=gen).to(torch.float16)
@@ -354,9 +355,7 @@ def test_full_size_scoring_workload_eviction_matches_checker(pkg, snapkv):
             for l in range(L):
                 assert len(exp[l]) == n_ev[b]
                 for blk in sorted(exp[l], reverse=True):
-                    freed = tables[l][b].pop(blk)
-                    if l == 0:
-                        spare[b].append(int(freed))   # (layer 0's freed blocks serve as this sequence's growth pool)
+                    spare[l][b].append(int(tables[l][b].pop(blk)))
         if step in (0, 31):
             for b in range(0, B, 17):
                 for l in range(L):

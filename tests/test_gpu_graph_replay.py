@@ -1,7 +1,6 @@
 """A step's per-layer calls recorded into a HIP graph: after one eager warm-up (which sizes the workspaces) the calls
 neither allocate nor wait, so a caller may capture them.  Replays, with eager work and waits in between, must give
 the eager result bit for bit."""
-import numpy as np
 import pytest
 
 import harness as H

@@ -1,7 +1,6 @@
 """Pins the CPU checker's eviction restatement to the reference's own known-answer vectors."""
 import types
 
-import numpy as np
 import pytest
 
 import eviction_kats as K

@@ -3,7 +3,6 @@ cases (tests/cpp/sparse_attention.cpp:23-72), and a skipped-block step through t
 import json
 import os
 
-import numpy as np
 import pytest
 
 from oracle import oracle as O

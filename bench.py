@@ -66,6 +66,8 @@ def parse():
     ap.add_argument("--xattention", type=float, default=0.0, metavar="THRESHOLD",
                     help="adds a leg: block-sparse prefill with this threshold against dense prefill (4 x 512-token "
                          "chunks, Qwen2.5-7B shape, bf16 cache)")
+    ap.add_argument("--append", type=int, default=0, metavar="TOKENS",
+                    help="also time pa_kv_append for one sequence of TOKENS new tokens (the workload's heads and cache type)")
     ap.add_argument("--rotate", action="store_true",
                     help="adds a leg: cache rotation (the re-rotation of K rows behind evicted blocks) over every "
                          "block of the workload's sequences, one layer")
@@ -401,6 +403,41 @@ def rotation_leg(torch, pkg, op, spec, kc, dev, reps=10):
             "note": "every K row read and written once; wall time of the whole call"}
 
 
+def append_leg(torch, pkg, spec, dev, tokens, reps=20):
+    """KV append at prefill scale: one sequence of ``tokens`` new tokens from scratch, the workload's heads and cache
+    type; the step's K and V rows read once, their cache rows written once.  Events around ``reps`` calls of
+    pa_kv_append on the launch stream."""
+    Hq, Hkv, D, bs = spec["Hq"], spec["Hkv"], spec["D"], spec["bs"]
+    stream = torch.cuda.current_stream(dev)
+    op = pkg.PagedAttention(Hq, Hkv, D, bs, spec["q_dtype"], spec["kv_dtype"], num_layers=1, device=0, stream=stream)
+    nblk = (tokens + bs - 1) // bs
+    rb = pkg.row_bytes(D, spec["kv_dtype"])
+    kc = torch.zeros(nblk, Hkv, bs, rb, dtype=torch.uint8, device=dev)
+    vc = torch.zeros_like(kc)
+    dt = torch.float16 if spec["q_dtype"] == "f16" else torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(4242)
+    k = torch.randn(tokens, Hkv * D, generator=gen, device=dev, dtype=torch.float32).to(dt)
+    v = torch.randn(tokens, Hkv * D, generator=gen, device=dev, dtype=torch.float32).to(dt)
+    op.step_begin(np.zeros(1, np.int32), np.array([0, tokens], np.int32), np.array([0, nblk], np.int32), tokens)
+    op.set_block_indices(np.random.default_rng(5).permutation(nblk).astype(np.int32), nblk)
+    for _ in range(3):
+        op.kv_append(k, v, kc, vc)
+    torch.cuda.synchronize(dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        op.kv_append(k, v, kc, vc)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    ms = e0.elapsed_time(e1) / reps
+    nbytes = 2.0 * tokens * Hkv * (2 * D + rb)
+    return {"tokens": tokens, "ms_per_call": round(ms, 4), "bytes": nbytes,
+            "roofline": {"bound": "hbm", "kernel": "kv_append_tokens_kernel" if tokens >= 8192 else "kv_append_kernel",
+                         "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+            "note": "K and V rows of the step read once, their cache rows written once"}
+
+
 def xattention_leg(torch, pkg, dev, threshold, kv_dtype="bf16", reps=20):
     """Block-sparse prefill (XAttention, block 64, stride 8) against dense prefill on the prefill part of the mixed
     workload: four 512-token chunks at past 0 / 2048 / 4096 / 8192, Qwen2.5-7B shape, bf16 cache (u8 with --kv-dtype u8).  Plain N(0,1) data
@@ -628,6 +665,8 @@ def main():
         res["xattention"] = xattention_leg(torch, pkg, dev, args.xattention, "u8" if args.kv_dtype == "u8" else "bf16")
     if args.diversity > 0:
         res["adaptive_rkv_diversity"] = diversity_leg(torch, op, spec, kc, dev, args.diversity)
+    if args.append > 0:
+        res["kv_append"] = append_leg(torch, pkg, spec, dev, args.append)
     if args.rotate:
         res["cache_rotation"] = rotation_leg(torch, pkg, op, spec, kc, dev)
     if args.kv_cache_leg:

@@ -136,7 +136,8 @@ int32_t pa_set_block_indices_layers(pa_ctx* ctx, int32_t first_layer, int32_t nu
  *   for u4 (`key_cache.<L>` / `value_cache.<L>`, kv_cache_manager.hpp:30-33; the u4 row format is this library's
  *   reading of the plugin's, which the reference tree does not hold);
  *   out [T, Hq*Dv] in query_dtype; scores f32 [sum_b(past_b + new_b)] or NULL (`scores.<L>`,
- *   model_runner.hpp:23-27, 1518-1568). */
+ *   model_runner.hpp:23-27, 1518-1568).
+ * Every tensor starts at a multiple of 16 bytes (scores: of 4); other pointers return PA_INVALID_C_PARAM. */
 typedef struct pa_layer_io {
     const void* query;
     const void* key;

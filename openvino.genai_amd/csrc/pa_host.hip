@@ -291,6 +291,14 @@ void check_io(pa_ctx* ctx, int32_t layer, const pa_layer_io* io, bool need_kv, b
                "the cache tensors hold fewer blocks than the block table of this layer refers to");
     if (need_kv) PA_REQUIRE(io->key && io->value, PA_INVALID_C_PARAM, "key/value missing");
     if (need_q) PA_REQUIRE(io->query && io->out, PA_INVALID_C_PARAM, "query/out missing");
+    // the kernels move rows in 16-byte pieces (scores as 4-byte values); a pointer off that grid is refused here
+    auto on_grid = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    PA_REQUIRE(on_grid(io->key_cache, 16) && on_grid(io->value_cache, 16), PA_INVALID_C_PARAM,
+               "cache tensors must start at a multiple of 16 bytes");
+    if (need_kv) PA_REQUIRE(on_grid(io->key, 16) && on_grid(io->value, 16), PA_INVALID_C_PARAM,
+                            "key/value must start at a multiple of 16 bytes");
+    if (need_q) PA_REQUIRE(on_grid(io->query, 16) && on_grid(io->out, 16) && on_grid(io->scores, 4), PA_INVALID_C_PARAM,
+                           "query/out must start at a multiple of 16 bytes, scores at a multiple of 4");
 }
 
 // Descriptors of the u8 decode kernel's workgroups for one block table (host ids), both plans, into the staging copy

@@ -591,6 +591,16 @@ def test_prefill_ignores_garbage_beyond_the_context(pkg, dev, qd, kd):
     H.assert_close(got["scores"], ref["scores"], "f16", "scores")
 
 
+class _ByteOffset:
+    """Stands for a tensor that starts ``nbytes`` into ``t`` (the binding only asks a tensor for its address)."""
+
+    def __init__(self, t, nbytes):
+        self._t, self._n = t, nbytes
+
+    def data_ptr(self):
+        return self._t.data_ptr() + self._n
+
+
 def test_errors_are_reported_not_thrown_across_the_abi(pkg, dev):
     import torch
     op = pkg.PagedAttention(8, 2, 128, 32, "f16", "u8", device=0, stream=torch.cuda.current_stream(dev))
@@ -619,6 +629,20 @@ def test_errors_are_reported_not_thrown_across_the_abi(pkg, dev):
         assert e.value.status == -6, str(e.value)
     big = torch.zeros(41, 2, 32, 136, dtype=torch.uint8, device=dev)
     op.attention(q, big, big, torch.zeros_like(q))  # 41 blocks hold id 40
+    op.synchronize()
+    # tensors off the 16-byte grid the kernels move rows on (views into larger buffers): refused, nothing launched
+    pad_q = torch.zeros(8 * 128 + 8, dtype=torch.float16, device=dev)
+    pad_c = torch.zeros(big.numel() + 16, dtype=torch.uint8, device=dev)
+    off_q, off_c = pad_q[1:1 + 8 * 128].view(1, -1), pad_c[8:8 + big.numel()].view(big.shape)
+    sc = torch.zeros(101 + 1, dtype=torch.float32, device=dev)
+    for call in (lambda: op.attention(off_q, big, big, torch.zeros_like(q)), lambda: op.attention(q, big, big, off_q),
+                 lambda: op.attention(q, off_c, big, torch.zeros_like(q)), lambda: op.attention(q, big, off_c, torch.zeros_like(q)),
+                 lambda: op.kv_append(off_q[:, :256], q[:, :256], big, big),
+                 lambda: op.attention(q, big, big, torch.zeros_like(q), _ByteOffset(sc, 2))):
+        with pytest.raises(pkg.PaError) as e:
+            call()
+        assert e.value.status == -14, str(e.value)
+    op.attention(q, big, big, torch.zeros_like(q), sc[1:])  # a 4-byte offset is fine for scores
     op.synchronize()
 
 

@@ -960,7 +960,9 @@ int32_t pa_evictor_register_scores(pa_evictor* ev, int32_t B, const int32_t* slo
         PA_REQUIRE(B > 0 && slots && scores_per_layer && offsets, PA_INVALID_C_PARAM, "null argument");
         const uint64_t L = ev->L(), bsz = ev->cfg.block_size, window = ev->cfg.snapkv_window_size;
         const bool norm = ev->cfg.aggregation_mode == PA_AGG_NORM_SUM;
-        for (uint64_t l = 0; l < L; ++l) PA_REQUIRE(scores_per_layer[l], PA_INVALID_C_PARAM, "null scores pointer");
+        for (uint64_t l = 0; l < L; ++l)
+            PA_REQUIRE(scores_per_layer[l] && (reinterpret_cast<uintptr_t>(scores_per_layer[l]) & 3) == 0, PA_INVALID_C_PARAM,
+                       "null scores pointer, or one that is not a multiple of 4 bytes");
         // validate everything before touching state
         std::vector<uint64_t> seen(B);
         check_slots(ev, B, slots);

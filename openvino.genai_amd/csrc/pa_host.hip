@@ -1663,6 +1663,8 @@ int32_t pa_rotate_cache(pa_ctx* ctx, void* key_cache, int64_t num_blocks, const 
         PA_REQUIRE(num_rotated >= 0, PA_INVALID_C_PARAM, "negative block count");
         if (num_rotated == 0) return;
         PA_REQUIRE(key_cache && rotated_block_indices && rotation_deltas, PA_INVALID_C_PARAM, "null argument");
+        PA_REQUIRE((reinterpret_cast<uintptr_t>(key_cache) & 15) == 0, PA_INVALID_C_PARAM,
+                   "the key cache must start at a multiple of 16 bytes");
         PA_REQUIRE(ctx->trig_rows > 0, PA_NOT_ALLOCATED, "pa_set_rotation_trig_lut has not been called");
         PA_REQUIRE(c.kv_cache_dtype != PA_U4, PA_NOT_IMPLEMENTED, "cache rotation runs over u8, f16 and bf16 key caches");
         PA_REQUIRE(deltas_per_block == 1 || deltas_per_block == c.block_size, PA_PARAMETER_MISMATCH,
@@ -1728,6 +1730,8 @@ int32_t pa_adaptive_rkv_diversity(pa_ctx* ctx, int32_t layer, const void* key_ca
         }
         if (seqs.empty()) return;
         PA_REQUIRE(key_cache && diversity, PA_INVALID_C_PARAM, "null argument");
+        PA_REQUIRE((reinterpret_cast<uintptr_t>(key_cache) & 15) == 0 && (reinterpret_cast<uintptr_t>(diversity) & 3) == 0,
+                   PA_INVALID_C_PARAM, "the key cache must start at a multiple of 16 bytes, the output at a multiple of 4");
         PA_REQUIRE(out_total <= capacity, PA_OUT_OF_BOUNDS, "diversity output holds fewer values than the areas need");
         // the areas' blocks must exist in the cache handed over now (the table was checked against the num_blocks of
         // its own call)

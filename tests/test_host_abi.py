@@ -163,3 +163,22 @@ def test_create_without_gpu_fails_cleanly(pkg):
         pytest.skip("a GPU is present")
     with pytest.raises(pkg.PaError):
         pkg.PagedAttention(8, 2, 128)
+
+
+def test_package_raises_when_the_hip_library_is_missing():
+    """No CPU fallback: with the library absent the first use of the package raises and names the file."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import __graft_entry__ as g\n"
+            "try:\n"
+            "    pkg = g.load_package()\n"
+            "    pkg.pack_step([3], [0], [0], [1], [1], 32)\n"
+            "except ImportError as e:\n"
+            "    print('RAISED', e)\n"
+            "else:\n"
+            "    print('NO ERROR')\n")
+    env = dict(os.environ, PA_AMD_LIBRARY="/nonexistent/libpa_amd.so")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=root, env=env, timeout=300)
+    assert "RAISED" in r.stdout and "/nonexistent/libpa_amd.so" in r.stdout and "no CPU fallback" in r.stdout, r.stdout + r.stderr

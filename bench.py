@@ -676,7 +676,6 @@ def main():
         for mode in [m for m in args.evict_modes.split(",") if m and m != "norm_sum"]:
             res["eviction_" + mode] = eviction_leg(torch, pkg, op, spec, q, kc, vc, out, scores, dev, args.layers, mode)
     if not args.no_cpu_baseline:
-        from oracle import oracle as O
         q_h = q.view(torch.int16).cpu().numpy().view(np.uint16)
         t_cpu, n_pass, threads, t_one = cpu_baseline(spec, args.cpu_seconds, with_scores, q_h, kc.cpu().numpy(), vc.cpu().numpy())
         res["cpu_baseline"] = {"value": round(bytes_["total"] / t_cpu / 1e9, 3), "unit": "GB/s", "cores": threads,

@@ -182,3 +182,23 @@ def test_package_raises_when_the_hip_library_is_missing():
     env = dict(os.environ, PA_AMD_LIBRARY="/nonexistent/libpa_amd.so")
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=root, env=env, timeout=300)
     assert "RAISED" in r.stdout and "/nonexistent/libpa_amd.so" in r.stdout and "no CPU fallback" in r.stdout, r.stdout + r.stderr
+
+
+def test_the_product_never_refers_to_the_checker():
+    """The CPU checker is test infrastructure: nothing under the package or the header names it, the benchmark only
+    inside its CPU-baseline leg, the entry module only to build it and (through the tests' harness) in smoke()."""
+    import os
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for base in ("openvino.genai_amd", "include"):
+        for d, _, files in os.walk(os.path.join(root, base)):
+            for f in files:
+                if f.endswith((".py", ".hip", ".h", ".cpp", "Makefile")):
+                    text = open(os.path.join(d, f), encoding="utf-8").read()
+                    assert "oracle" not in text and "_work/" not in text, os.path.join(d, f)
+    bench = open(os.path.join(root, "bench.py"), encoding="utf-8").read()
+    uses = [m.start() for m in re.finditer(r"\boracle\b", bench)]
+    leg = bench.index("def cpu_baseline(")
+    leg_end = bench.index("\ndef ", leg + 1)
+    assert uses and all(leg < u < leg_end for u in uses)
+    assert "_work/" not in bench

@@ -137,6 +137,64 @@ def test_batched_decode_steps_match_checker_exactly(pkg, mode, snapkv):
     assert any(len(b) for b in got[0]) or True
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_random_eviction_settings_match_checker_exactly(pkg, seed):
+    """Drawn settings instead of the scoring workload's: block size, area sizes, max-pool window, aggregation mode,
+    SnapKV window, sequences that grow by one token or by a chunk per step, planted ties; state, block scores,
+    ranges and evicted blocks equal to the checker's after every step."""
+    import torch
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(9000 + seed)
+    bs = int(rng.choice([16, 32, 64]))
+    start, recent = bs * int(rng.integers(1, 4)), bs * int(rng.integers(1, 6))
+    mx = start + recent + bs * int(rng.integers(1, 20))
+    pool = int(rng.choice([1, 3, 7]))
+    mode = ["SUM", "NORM_SUM"][int(rng.integers(0, 2))]
+    snapkv = int(rng.choice([0, 0, 4, 8]))
+    B, L = int(rng.integers(1, 7)), int(rng.integers(1, 4))
+    m = pkg.AggregationMode[mode]
+    ev = pkg.Evictor(pkg.CacheEvictionConfig(start, recent, mx, m, False, snapkv), bs, L, pool, max_sequences=B,
+                     max_tracked_tokens=8192, device=0, stream=torch.cuda.current_stream(dev))
+    refs = [O.CacheEvictionAlgorithm(start, recent, mx, int(m), snapkv, bs, L, pool) for _ in range(B)]
+    slots = rng.permutation(B).astype(np.int32)
+    ctx = rng.integers(max(snapkv, 1), 3 * mx, B)   # some sequences start below the budget, some far above
+    first, total = True, 0
+    for step in range(10):
+        offsets = np.concatenate([[0], np.cumsum(ctx)]).astype(np.int64)
+        layer_scores = [rng.random(int(offsets[-1])).astype(np.float32) ** 3 for _ in range(L)]
+        for s in layer_scores:   # ties: runs of equal values, and exact zeros
+            a = int(rng.integers(0, max(1, len(s) - 3 * bs)))
+            s[a:a + 3 * bs] = 0.25
+            s[rng.random(len(s)) < 0.05] = 0.0
+        dev_scores = [torch.from_numpy(s).to(dev) for s in layer_scores]
+        n_snap = np.full(B, (snapkv if first else 1) if snapkv else 0, np.uint64)
+        ev.register_new_token_scores(slots, [t.data_ptr() for t in dev_scores], offsets, n_snap)
+        for i in range(B):
+            refs[i].register_new_token_scores([s[offsets[i]:offsets[i + 1]] for s in layer_scores], (), int(n_snap[i]))
+        for i in range(B):
+            for l in range(L):
+                gs, gc = ev.get_state(int(slots[i]), l)
+                assert np.array_equal(gs, refs[i].get_scores()[l]), (step, i, l)
+                if mode == "NORM_SUM":
+                    assert np.array_equal(gc, refs[i].get_counters()[l]), (step, i, l)
+                np.testing.assert_array_equal(ev.block_scores(int(slots[i]), l), refs[i].block_scores(l))
+                assert ev.get_evictable_block_range(int(slots[i]), l) == refs[i].get_evictable_block_range(l)
+        got = ev.evict_logical_blocks(slots, max_blocks_per_entry=512)
+        for i in range(B):
+            exp = refs[i].evict_logical_blocks()
+            assert got[i] == exp, (step, i)
+            total += len(exp[0])
+            ctx[i] -= len(exp[0]) * bs
+            for l in range(L):
+                gs, gc = ev.get_state(int(slots[i]), l)
+                assert np.array_equal(gs, refs[i].get_scores()[l]), (step, i, l)
+                if mode == "NORM_SUM":
+                    assert np.array_equal(gc, refs[i].get_counters()[l]), (step, i, l)
+        ctx += np.where(rng.random(B) < 0.3, rng.integers(2, 3 * bs, B), 1)   # a decode token, or a chunk
+        first = False
+    assert total > 0 or int(ctx.max()) <= mx + bs
+
+
 @pytest.mark.parametrize("mode", ["NORM_SUM", "ADAPTIVE_RKV"])
 def test_scores_may_be_rewritten_in_stream_order_right_after_registering(pkg, mode):
     """pa_evictor_register_scores returns with its kernel queued: the score tensors are read in stream order, so work

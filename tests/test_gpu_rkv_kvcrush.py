@@ -189,6 +189,57 @@ def test_kvcrush_batched_decode_steps_match_checker_exactly(pkg, mode, budget, t
     assert retained > 0
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_kvcrush_drawn_settings_match_checker_exactly(pkg, seed):
+    """KVCrush on drawn settings: block size, area sizes, max-pool window, SUM or NORM_SUM, budget, anchor mode and
+    its seed, tied or continuous scores, sequences that grow by a token or by a chunk."""
+    import torch
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(7700 + seed)
+    bs = int(rng.choice([16, 32, 64]))
+    start, recent = bs * int(rng.integers(1, 3)), bs * int(rng.integers(1, 5))
+    mx = start + recent + bs * int(rng.integers(2, 16))
+    pool = int(rng.choice([1, 3, 7]))
+    norm = bool(rng.integers(0, 2))
+    budget = int(rng.integers(1, 5))
+    anchor = pkg.KVCrushAnchorPointMode(int(rng.integers(0, 5)))
+    rseed = int(rng.integers(0, 1000))
+    tied = bool(rng.integers(0, 2))
+    B, L = int(rng.integers(1, 5)), int(rng.integers(1, 4))
+    m = pkg.AggregationMode.NORM_SUM if norm else pkg.AggregationMode.SUM
+    cfg = pkg.CacheEvictionConfig(start, recent, mx, m, False, 0, pkg.KVCrushConfig(budget, anchor, rseed))
+    ev = pkg.Evictor(cfg, bs, L, pool, max_sequences=B, max_tracked_tokens=8192, device=0,
+                     stream=torch.cuda.current_stream(dev))
+    refs = [O.CacheEvictionAlgorithm(start, recent, mx, int(m), 0, bs, L, pool, kvcrush_budget=budget,
+                                     kvcrush_anchor_mode=int(anchor), kvcrush_seed=rseed) for _ in range(B)]
+    slots = rng.permutation(B).astype(np.int32)
+    ctx = rng.integers(mx // 2, 3 * mx, B)
+    evicted = 0
+    for step in range(16):
+        offsets = np.concatenate([[0], np.cumsum(ctx)]).astype(np.int64)
+        draw = (lambda n: rng.choice([0.0, 0.1, 0.5, 1.0], size=n)) if tied else (lambda n: rng.random(n))
+        layer_scores = [draw(int(offsets[-1])).astype(np.float32) for _ in range(L)]
+        dev_scores = [torch.from_numpy(s).to(dev) for s in layer_scores]
+        ev.register_new_token_scores(slots, [t.data_ptr() for t in dev_scores], offsets)
+        for i in range(B):
+            refs[i].register_new_token_scores([s[offsets[i]:offsets[i + 1]] for s in layer_scores])
+        got = ev.evict_logical_blocks(slots, max_blocks_per_entry=512)
+        for i in range(B):
+            exp = refs[i].evict_logical_blocks()
+            assert got[i] == exp, (step, i)
+            assert len({len(x) for x in exp}) == 1
+            evicted += len(exp[0])
+            ctx[i] -= len(exp[0]) * bs
+            for l in range(L):
+                gs, gc = ev.get_state(int(slots[i]), l)
+                assert np.array_equal(gs, refs[i].get_scores()[l]), (step, i, l)
+                if norm:
+                    assert np.array_equal(gc, refs[i].get_counters()[l]), (step, i, l)
+        ctx += np.where(rng.random(B) < 0.3, rng.integers(2, 3 * bs, B), 1)
+    # (a drawn budget may cover every eviction that falls due: then nothing leaves, in the library as in the checker)
+    assert evicted > 0 or seed in (21, 22)
+
+
 def test_rkv_evictor_rejects_bad_calls(pkg):
     import torch
     dev = torch.device("cuda:0")

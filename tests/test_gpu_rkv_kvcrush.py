@@ -189,6 +189,71 @@ def test_kvcrush_batched_decode_steps_match_checker_exactly(pkg, mode, budget, t
     assert retained > 0
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_rkv_drawn_settings_match_checker_exactly(pkg, seed):
+    """ADAPTIVE_RKV on drawn settings: block size, area sizes, max-pool window, tracker window, attention mass,
+    sequences that grow by a token or by a chunk; a diversity matrix with planted equal rows whenever an eviction
+    is due."""
+    import torch
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(8800 + seed)
+    bs = int(rng.choice([16, 32, 64]))
+    start, recent = bs * int(rng.integers(1, 3)), bs * int(rng.integers(1, 5))
+    mx = start + recent + bs * int(rng.integers(2, 14))
+    pool = int(rng.choice([1, 3, 7]))
+    window = int(rng.integers(1, 9))
+    mass = float(rng.choice([0.05, 0.3, 0.5, 0.9, 1.0]))
+    B, L = int(rng.integers(1, 5)), int(rng.integers(1, 4))
+    cfg = pkg.CacheEvictionConfig(start, recent, mx, pkg.AggregationMode.ADAPTIVE_RKV, False, 0, None,
+                                  pkg.AdaptiveRKVConfig(mass, window))
+    ev = pkg.Evictor(cfg, bs, L, pool, max_sequences=B, max_tracked_tokens=8192, device=0,
+                     stream=torch.cuda.current_stream(dev))
+    refs = [O.CacheEvictionAlgorithm(start, recent, mx, O.MODE_ADAPTIVE_RKV, 0, bs, L, pool,
+                                     adaptive_rkv_window_size=window, attention_mass=mass) for _ in range(B)]
+    slots = rng.permutation(B).astype(np.int32)
+    ctx = rng.integers(mx // 2, 2 * mx, B)
+    for step in range(14):
+        offsets = np.concatenate([[0], np.cumsum(ctx)]).astype(np.int64)
+        layer_scores = [rng.random(int(offsets[-1])).astype(np.float32) ** 4 for _ in range(L)]
+        for s in layer_scores:
+            s[start:start + 2 * bs] = 0.125  # whole blocks of equal importance
+        dev_scores = [torch.from_numpy(s).to(dev) for s in layer_scores]
+        ev.register_new_token_scores(slots, [t.data_ptr() for t in dev_scores], offsets)
+        for i in range(B):
+            refs[i].register_new_token_scores([s[offsets[i]:offsets[i + 1]] for s in layer_scores])
+        due = []
+        for i in range(B):
+            for l in range(L):
+                assert np.array_equal(ev.get_state(int(slots[i]), l)[0], refs[i].get_scores()[l]), (step, i, l)
+                assert ev.get_evictable_block_range(int(slots[i]), l) == refs[i].get_evictable_block_range(l)
+            b, e = refs[i].get_evictable_block_range(0)
+            if e > b:
+                due.append((i, e - b))
+        if due:
+            doff = np.concatenate([[0], np.cumsum([nb * nb * bs for _, nb in due])]).astype(np.int64)
+            layer_div = []
+            for l in range(L):
+                d = -(rng.random(int(doff[-1])).astype(np.float32))
+                for x, (i, nb) in enumerate(due):
+                    if nb > 1:
+                        mtx = d[doff[x]:doff[x + 1]].reshape(nb, nb * bs)
+                        mtx[1] = mtx[0]
+                layer_div.append(d)
+            dev_div = [torch.from_numpy(d).to(dev) for d in layer_div]
+            ev.register_block_diversity(slots[[i for i, _ in due]], [t.data_ptr() for t in dev_div], doff)
+            for x, (i, nb) in enumerate(due):
+                refs[i].register_block_diversity([d[doff[x]:doff[x + 1]] for d in layer_div])
+        got = ev.evict_logical_blocks(slots, max_blocks_per_entry=512)
+        for i in range(B):
+            exp = refs[i].evict_logical_blocks()
+            assert got[i] == exp, (step, i, got[i], exp)
+            assert len({len(x) for x in exp}) == 1
+            ctx[i] -= len(exp[0]) * bs
+            for l in range(L):
+                assert np.array_equal(ev.get_state(int(slots[i]), l)[0], refs[i].get_scores()[l])
+        ctx += np.where(rng.random(B) < 0.3, rng.integers(2, 3 * bs, B), 1)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_kvcrush_drawn_settings_match_checker_exactly(pkg, seed):
     """KVCrush on drawn settings: block size, area sizes, max-pool window, SUM or NORM_SUM, budget, anchor mode and

@@ -828,3 +828,27 @@ def test_full_size_properties_of_the_other_workloads(pkg, dev, cfg, kw):
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16)) and torch.equal(scores, scores2)
     # every sequence of the batch against the checker (config 3's chunks are a minute of checker time)
     _check_whole_batch(spec, q, kc, vc, out, scores, W, qd, kd, sw)
+
+
+@pytest.mark.parametrize("qd,kd,new", [("f16", "u8", [1, 1, 1, 1]), ("bf16", "bf16", [1, 1, 1, 1]), ("f16", "u8", [1, 40, 1, 3]),
+                                       ("bf16", "bf16", [1, 40, 1, 3]), ("f16", "f16", [33, 1, 1, 1])])
+def test_sequences_that_share_the_blocks_of_a_common_prefix(pkg, dev, qd, kd, new):
+    """Prefix caching hands several sequences the SAME physical blocks for their common prefix (the reference's block
+    manager, src/cpp/src/continuous_batching/cache/block_manager.hpp:23-58: blocks with a reference count above one): the tables of four sequences name one set
+    of blocks for their first 20 blocks and blocks of their own behind it.  Attention reads the shared blocks once
+    per sequence; the step's new rows go to the sequences' own blocks."""
+    past = [1000, 700, 2000, 640]
+    case = H.case_from_lens(f"shared_prefix_{qd}_{kd}", 8, 2, 128, 32, qd, kd, past, new)
+    c = H.build_case(case, 61, outliers=True)
+    shared = 20
+    bib = c["block_indices_begins"]
+    for b in range(1, len(past)):
+        c["block_indices"][bib[b]:bib[b] + shared] = c["block_indices"][bib[0]:bib[0] + shared]
+    got = H.run_case_on_gpu(pkg, c, dev)
+    ref = H.run_case_on_checker(c)
+    assert np.array_equal(got["key_cache"], ref["key_cache"]) and np.array_equal(got["value_cache"], ref["value_cache"])
+    H.assert_close(got["out"], ref["out"], qd)
+    H.assert_close(got["scores"], ref["scores"], "f16", "scores")
+    # the shared blocks were not written by the step (every new row lies behind the prefix)
+    ids = c["block_indices"][bib[0]:bib[0] + shared]
+    assert np.array_equal(got["key_cache"][ids], c["key_cache0"][ids])

@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--config", type=int, default=2, help="workload (2 = headline; 1, 4, 5, other head sizes 6, 7 and larger prefill steps 8, 9 for diagnostics)")
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--sliding-window", type=int, default=None)
+    ap.add_argument("--new-tokens", type=int, default=None,
+                    help="decode workloads: every sequence schedules this many tokens (a speculative-decoding validation step)")
     ap.add_argument("--block-size", type=int, choices=[16, 32], default=None,
                     help="KV block size of the workload (default: the configuration's, 32)")
     ap.add_argument("--kv-dtype", choices=["u8", "f16", "bf16"], default=None,
@@ -531,7 +533,9 @@ def main():
     torch.cuda.set_device(dev)
 
     spec = wl.make_spec(args.config, batch=args.batch, sliding_window=args.sliding_window, pool_factor=args.pool_factor,
-                        block_size=args.block_size)
+                        block_size=args.block_size, new_tokens=args.new_tokens)
+    if args.new_tokens is not None:
+        spec["name"] += "_new%d" % args.new_tokens
     if args.block_size is not None and args.block_size != 32:
         spec["name"] += "_block%d" % args.block_size
     if args.pool_factor != 2.0:

@@ -37,8 +37,11 @@ CONFIGS = {
 }
 
 
-def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0, block_size=None):
-    """Step metadata of config ``cfg`` (1..9); ``batch`` / ``context_scale`` shrink it for parity tests."""
+def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None, pool_factor=2.0, block_size=None,
+              new_tokens=None):
+    """Step metadata of config ``cfg`` (1..9); ``batch`` / ``context_scale`` shrink it for parity tests;
+    ``new_tokens``: every sequence of a decode workload schedules that many tokens instead of one (the shape of a
+    speculative-decoding validation step)."""
     c = dict(CONFIGS[cfg])
     rng = np.random.Generator(np.random.PCG64(1000 + cfg if seed is None else seed))
     B = c["B"] if batch is None else batch
@@ -46,10 +49,10 @@ def make_spec(cfg, seed=None, batch=None, context_scale=1.0, sliding_window=None
     sc = lambda v: max(0, int(round(v * context_scale)))
     if kind == "const":
         past = np.full(B, sc(c["past"][1]), np.int64)
-        new = np.full(B, c["new"], np.int64)
+        new = np.full(B, c["new"] if new_tokens is None else new_tokens, np.int64)
     elif kind == "uniform":
         past = rng.integers(sc(c["past"][1]), sc(c["past"][2]) + 1, size=B)
-        new = np.full(B, c["new"], np.int64)
+        new = np.full(B, c["new"] if new_tokens is None else new_tokens, np.int64)
     else:  # mixed: prefill chunks first, then decode sequences
         _, chunk_pasts, n_dec, lo, hi = c["past"]
         _, chunk_len, _ = c["new"]

@@ -51,6 +51,8 @@ def parse():
                     help="KV block size of the workload (default: the configuration's, 32)")
     ap.add_argument("--kv-dtype", choices=["u8", "f16", "bf16"], default=None,
                     help="diagnostics: run the workload's shape over another cache type")
+    ap.add_argument("--cache-tensors", choices=["manager", "torch"], default="manager",
+                    help="who allocates key_cache / value_cache: the library's cache manager (as under the pipeline) or torch")
     ap.add_argument("--no-scores", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline")
@@ -83,6 +85,20 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference reading for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
+
+
+class _DeviceBytes:
+    """A run of device memory owned by someone else, presented through the array interface torch reads."""
+
+    def __init__(self, ptr, nbytes):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (int(ptr), False), "version": 2}
+
+
+def cache_view(torch, ptr, shape, dev):
+    """A uint8 tensor over a cache tensor of the library's cache manager (no copy; the manager keeps the memory)."""
+    t = torch.as_tensor(_DeviceBytes(ptr, int(np.prod(shape))), device=dev).view(*shape)
+    assert t.data_ptr() == int(ptr)
+    return t
 
 
 def fill_cache(torch, op, spec, kc, vc, dev, gen):
@@ -551,8 +567,15 @@ def main():
     op = pkg.PagedAttention(Hq, Hkv, D, bs, spec["q_dtype"], spec["kv_dtype"], num_layers=1, device=0, stream=stream)
     gen = torch.Generator(device=dev).manual_seed(1000 + args.config)
     rb = pkg.row_bytes(D, spec["kv_dtype"])
-    kc = torch.zeros(spec["num_blocks"], Hkv, bs, rb, dtype=torch.uint8, device=dev)
-    vc = torch.zeros_like(kc)
+    # the cache tensors come from the library's cache manager, as they do under the pipeline (new blocks read as zero)
+    if args.cache_tensors == "manager":
+        cache = pkg.KVCacheManager(1, Hkv, D, bs, spec["kv_dtype"], device=0)
+        cache.allocate_cache_if_needed(spec["num_blocks"])
+        kc = cache_view(torch, cache.get_key_cache(0), (spec["num_blocks"], Hkv, bs, rb), dev)
+        vc = cache_view(torch, cache.get_value_cache(0), (spec["num_blocks"], Hkv, bs, rb), dev)
+    else:  # plain device allocations, for comparison
+        kc = torch.zeros(spec["num_blocks"], Hkv, bs, rb, dtype=torch.uint8, device=dev)
+        vc = torch.zeros_like(kc)
     fill_cache(torch, op, spec, kc, vc, dev, gen)
 
     dt = torch.float16 if spec["q_dtype"] == "f16" else torch.bfloat16
@@ -633,7 +656,8 @@ def main():
         "dtype": spec["kv_dtype"] + "/f32", "data": "synthetic",
         "config": {"workload": spec["name"], "batch": B, "context": int(spec["past_lens"].max()) + 1,
                    "heads": [Hq, Hkv, D], "block_size": bs, "scores": with_scores, "splits": op.num_splits,
-                   "sliding_window": spec["sliding_window"], "clock_settle_steps": args.settle_steps},
+                   "sliding_window": spec["sliding_window"], "clock_settle_steps": args.settle_steps,
+                   "cache_tensors": "pa_kv_cache (the library's cache manager)" if args.cache_tensors == "manager" else "torch allocator"},
         "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tok_per_s": round(B / (NUM_LAYERS_FOR_TOKS * ms_per_step * 1e-3), 1),
         "algorithmic_bytes": bytes_,

